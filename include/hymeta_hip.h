@@ -29,7 +29,10 @@
  *    version 3: hymeta_gla_decode_args ends with qkv_x_scale / qkv_w_scale;
  *    version 4: the recurrent / biased-attention building blocks;
  *    version 5: hymeta_sink_attention_args ends with sink_logits / kv_layout, hymeta_moe_gemm_any_args with
- *    act_limit / act_alpha; the post-norm, latent- and linear-attention building blocks at the end of this file).
+ *    act_limit / act_alpha; the post-norm, latent- and linear-attention building blocks at the end of this file;
+ *    version 6: hymeta_sink_attention_args ends with keep_first, hymeta_moe_route_sigmoid_args with router_bias /
+ *    score_mode; HYMETA_KV_SHARED_KEY, HYMETA_GLU_RELU2, HYMETA_ACT_SILU_MUL / HYMETA_ACT_RELU2; the hyper-connection
+ *    and talking-heads building blocks at the end of this file).
  *  - Every argument struct starts with `uint32_t struct_size`, which the caller
  *    sets to sizeof(the struct) of ITS declaration.  An entry point returns
  *    HYMETA_ERR_INVALID_ARG, before it reads any other field, when the value
@@ -47,7 +50,7 @@
 extern "C" {
 #endif
 
-#define HYMETA_ABI_VERSION 5
+#define HYMETA_ABI_VERSION 6
 
 typedef void* hymeta_stream_t;
 
@@ -1180,8 +1183,13 @@ enum hymeta_bias_mode { HYMETA_BIAS_NONE = 0, HYMETA_BIAS_LOG_DISTANCE = 1 };
  * latent shared by keys and values followed by a rotated key part: hymeta_latent_kv_prep); v_dim <= head_dim.  With
  * VALUE_IN_KEY bf16 rows with v_dim 64 or 128 and head_dim = v_dim + 32 or v_dim + 64 run on the matrix cores (the
  * kernels of KEY_THEN_VALUE with another staging of the tiles), and so do v_dim 256 / 384 / 512 with head_dim = v_dim + 64,
- * as 2 / 3 / 4 launches over value slices of 128; other sizes a wave per (row, head). */
-enum hymeta_kv_layout { HYMETA_KV_KEY_THEN_VALUE = 0, HYMETA_KV_VALUE_IN_KEY = 1 };
+ * as 2 / 3 / 4 launches over value slices of 128; other sizes a wave per (row, head).
+ * SHARED_KEY: a row is ONE key of head_dim elements that every query head reads, followed by num_kv_heads values of
+ * v_dim elements; query head h reads value h / (num_heads / num_kv_heads) (hymeta_talk_qkv_prep: queries that were
+ * mixed across heads against the concatenated keys of the key/value heads).  bf16 rows with head_dim 128 / 256 / 512 and
+ * v_dim 64 / 128 run on the matrix cores.
+ * keep_first (with window_left >= 0): keys j < keep_first stay visible to every later query, at their own positions. */
+enum hymeta_kv_layout { HYMETA_KV_KEY_THEN_VALUE = 0, HYMETA_KV_VALUE_IN_KEY = 1, HYMETA_KV_SHARED_KEY = 2 };
 typedef struct hymeta_sink_attention_args {
   uint32_t struct_size;
   const void* q;               /* act_dtype [num_tokens, num_heads, head_dim], strides q_stride_t / head_dim */
@@ -1200,6 +1208,7 @@ typedef struct hymeta_sink_attention_args {
   int64_t num_blocks, q_stride_t, block_table_stride;
   const float* sink_logits;    /* [num_heads] or NULL: the sink's score per head (NULL: 0); read when sink != 0 */
   int32_t kv_layout;           /* enum hymeta_kv_layout */
+  int32_t keep_first;          /* >= 0; read when window_left >= 0 */
 } hymeta_sink_attention_args;
 size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t num_kv_heads, int32_t v_dim,
                                              int32_t max_seq_len);
@@ -1228,7 +1237,8 @@ int hymeta_moe_route_table(const hymeta_moe_route_table_args* args, hymeta_strea
  * gated != 0: W[e] is [2 N, K] (gate rows, then up rows) and out[slot, n] = silu(gate_n) * up_n (HYMETA_GLU_SILU), or
  * g sigmoid(act_alpha g) (u + 1) with g = min(gate_n, act_limit), u = clamp(up_n, -act_limit, act_limit)
  * (HYMETA_GLU_CLAMPED).  row_scale as in hymeta_moe_gemm. */
-enum hymeta_glu_mode { HYMETA_GLU_NONE = 0, HYMETA_GLU_SILU = 1, HYMETA_GLU_CLAMPED = 2 };
+/* HYMETA_GLU_RELU2: not gated (W[e] is [N, K]); out[slot, n] = max(x W^T, 0)^2. */
+enum hymeta_glu_mode { HYMETA_GLU_NONE = 0, HYMETA_GLU_SILU = 1, HYMETA_GLU_CLAMPED = 2, HYMETA_GLU_RELU2 = 3 };
 typedef struct hymeta_moe_gemm_any_args {
   uint32_t struct_size;
   const void* x;               /* act_dtype rows of K */
@@ -1378,8 +1388,11 @@ int hymeta_gated_rms_norm(const hymeta_gated_rms_norm_args* args, hymeta_stream_
  *                           limit), out = g sigmoid(alpha g) (u + 1)
  *   HYMETA_ACT_XIELU        x [rows, n]: z > 0: a_pos z^2 + z / 2;  z <= 0: a_neg (exp(z) - 1 - z) + z / 2
  *   HYMETA_ACT_SIGMOID_MUL  x [rows, n], gate [rows, n]: out = x * sigmoid(gate)
+ *   HYMETA_ACT_SILU_MUL     x [rows, 2 n] (gate columns, then up columns): out = gate sigmoid(gate) up
+ *   HYMETA_ACT_RELU2        x [rows, n]: out = max(x, 0)^2
  * num_rows_dev: optional device count of the rows in use; NULL: num_rows. */
-enum hymeta_act_kind { HYMETA_ACT_CLAMPED_GLU = 0, HYMETA_ACT_XIELU = 1, HYMETA_ACT_SIGMOID_MUL = 2 };
+enum hymeta_act_kind { HYMETA_ACT_CLAMPED_GLU = 0, HYMETA_ACT_XIELU = 1, HYMETA_ACT_SIGMOID_MUL = 2, HYMETA_ACT_SILU_MUL = 3,
+                       HYMETA_ACT_RELU2 = 4 };
 typedef struct hymeta_activation_args {
   uint32_t struct_size;
   const void* x;               /* [rows, n or 2 n], row stride x_stride */
@@ -1392,9 +1405,11 @@ typedef struct hymeta_activation_args {
 } hymeta_activation_args;
 int hymeta_activation(const hymeta_activation_args* args, hymeta_stream_t stream);
 
-/* Router of a mixture of experts with sigmoid scores: logits = x router_weight^T in fp32, s = sigmoid(logits), the top_k
- * largest s are chosen (the lower expert on a tie), their weights are s / (sum of the chosen s + 1e-20) * scale.
+/* Router of a mixture of experts: logits = x router_weight^T (+ router_bias) in fp32; the top_k largest are chosen (the
+ * lower expert on a tie).  HYMETA_ROUTE_SIGMOID_SUM: s = sigmoid(logits), weights s / (sum of the chosen s + 1e-20) * scale.
+ * HYMETA_ROUTE_SOFTMAX_CHOSEN: weights = softmax over the chosen logits alone, times scale.
  * Writes what hymeta_moe_route writes.  num_experts <= HYMETA_MOE_TABLE_MAX_EXPERTS. */
+enum hymeta_route_mode { HYMETA_ROUTE_SIGMOID_SUM = 0, HYMETA_ROUTE_SOFTMAX_CHOSEN = 1 };
 typedef struct hymeta_moe_route_sigmoid_args {
   uint32_t struct_size;
   const void* x;               /* act_dtype [num_tokens, hidden], row stride x_stride_t */
@@ -1407,8 +1422,87 @@ typedef struct hymeta_moe_route_sigmoid_args {
   int32_t num_tokens, num_experts, top_k, hidden, act_dtype;
   float scale;
   int64_t x_stride_t;
+  const float* router_bias;    /* [num_experts] or NULL */
+  int32_t score_mode;          /* enum hymeta_route_mode */
 } hymeta_moe_route_sigmoid_args;
 int hymeta_moe_route_sigmoid(const hymeta_moe_route_sigmoid_args* args, hymeta_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Building blocks of pre-norm designs with several residual streams (hyper-connections) and attention whose scores
+ * are mixed across heads before the softmax.
+ * ---------------------------------------------------------------------- */
+
+/* Start of the residual streams: out[t, c, :] = norm(table[token_t] + pair_table[row_t]) for every copy c, fp32.
+ *   row_t = (previous token * mul_prev + token_t * mul_cur) mod buckets; a sequence's first token reads row `buckets`.
+ * The previous token of a portion's first row is sequence state: prev_token [slots] int32, read where context_lens > 0
+ * and rewritten with the portion's last token (by a first, tiny launch, so that no row reads a rewritten state).
+ * norm: layer norm over the row, (x - mean) / sqrt(var + eps) * norm_weight (NULL: no norm).  pair_table NULL: no pair
+ * rows.  first_rows: int32 scratch [num_seqs].  width <= 8192. */
+typedef struct hymeta_embed_pair_args {
+  uint32_t struct_size;
+  const int64_t* token_ids;    /* [num_tokens] */
+  const void* table;           /* act_dtype [vocab, width] */
+  const void* pair_table;      /* act_dtype [buckets + 1, width] or NULL */
+  const float* norm_weight;    /* [width] or NULL */
+  float* out;                  /* [num_tokens, copies, width] */
+  int32_t* prev_token;         /* [slots] */
+  int32_t* first_rows;         /* scratch [num_seqs] */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] */
+  const int32_t* context_lens;     /* [num_seqs] */
+  const int32_t* slot_idx;         /* [num_seqs] */
+  int32_t num_tokens, num_seqs, width, vocab, copies, act_dtype;
+  int64_t buckets, mul_prev, mul_cur;
+  float eps;
+} hymeta_embed_pair_args;
+int hymeta_embed_pair(const hymeta_embed_pair_args* args, hymeta_stream_t stream);
+
+/* One step of a set of residual streams x [num_tokens, streams, width] fp32, in place, one launch:
+ *   (y != NULL)      x_t <- sum_s mix[s, t] x_s + out_w[t] * y        all streams at once from the old ones
+ *   (h_out != NULL)  h = norm(sum_s in_w[s] x_s)                     from the new streams, act_dtype
+ * norm: layer norm times norm_weight (norm_weight NULL: the weighted sum itself).  One stream with mix = out_w = in_w =
+ * 1 is the plain residual add followed by the next sublayer's norm.  streams <= 8, width <= 8192. */
+typedef struct hymeta_hyper_stream_args {
+  uint32_t struct_size;
+  float* x;                    /* [num_tokens, streams, width] */
+  const void* y;               /* act_dtype [num_tokens, width], row stride y_stride_t; or NULL */
+  const float* mix;            /* [streams, streams], indexed [from, to] (with y) */
+  const float* out_w;          /* [streams] (with y) */
+  const float* in_w;           /* [streams] (with h_out) */
+  const float* norm_weight;    /* [width] or NULL */
+  void* h_out;                 /* act_dtype [num_tokens, width] contiguous; or NULL */
+  int32_t num_tokens, streams, width, act_dtype;
+  float eps;
+  int64_t y_stride_t;
+} hymeta_hyper_stream_args;
+#define HYMETA_MAX_STREAMS 8
+int hymeta_hyper_stream(const hymeta_hyper_stream_args* args, hymeta_stream_t stream);
+
+/* Between the fused q | k | v projection and hymeta_sink_attention with HYMETA_KV_SHARED_KEY, per token, one launch:
+ *   q <- rms_norm over all H * D query columns at once (times q_weight), k likewise over its G * D columns;
+ *   the first rot_dims dimensions of every head turn in interleaved pairs (2i, 2i + 1) by position * rot_freqs[i];
+ *   v <- (1 - v_blend) v + v_blend v_other (v_other != NULL);
+ *   the cache row at slot_mapping[t] <- (k of all G heads, v of all G heads);
+ *   q_out[t, h, g * D + d] = sum over the query heads j of group g of talk[h, j] q[j, d]:
+ * since scores mixed across heads, sum_j talk[h, j] (q_j . k_g(j)), are linear in the queries, they equal q_out[h] . (the
+ * concatenated keys).  All statistics, angles and sums are fp32 (angles are reduced in double precision). */
+typedef struct hymeta_talk_qkv_prep_args {
+  uint32_t struct_size;
+  const void* qkv;             /* act_dtype [num_tokens, H * D + G * D + G * Dv], row stride qkv_stride_t */
+  const float* q_weight;       /* [H * D] */
+  const float* k_weight;       /* [G * D] */
+  const float* talk;           /* [H, H] */
+  const double* rot_freqs;     /* [rot_dims / 2] */
+  const void* v_other;         /* act_dtype [num_tokens, G * Dv], row stride v_other_stride_t; or NULL */
+  void* q_out;                 /* act_dtype [num_tokens, H, G * D] contiguous */
+  void* kv_cache;              /* act_dtype rows of G * D + G * Dv */
+  const int64_t* slot_mapping; /* [num_tokens] */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] */
+  const int32_t* seq_lens;         /* [num_seqs] */
+  int32_t num_tokens, num_seqs, num_heads, num_kv_heads, head_dim, v_dim, rot_dims, block_size, act_dtype;
+  float eps, v_blend;
+  int64_t num_blocks, qkv_stride_t, v_other_stride_t;
+} hymeta_talk_qkv_prep_args;
+int hymeta_talk_qkv_prep(const hymeta_talk_qkv_prep_args* args, hymeta_stream_t stream);
 
 #ifdef __cplusplus
 }

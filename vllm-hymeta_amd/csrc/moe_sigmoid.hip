@@ -1,5 +1,5 @@
-// Router of a mixture of experts with sigmoid scores: fp32 logits from the rows and the router's matrix, the top_k
-// largest scores, weights normalised over the chosen and scaled; then the counting sort by expert that the grouped
+// Router of a mixture of experts: fp32 logits from the rows and the router's matrix (and bias), the top_k largest
+// (sigmoid scores normalised over the chosen and scaled, or a softmax over the chosen logits alone); then the counting sort by expert that the grouped
 // GEMMs of the routed block read.
 #include "act_types.h"
 
@@ -23,6 +23,7 @@ __global__ __launch_bounds__(256) void moe_scores_topk_kernel(hymeta_moe_route_s
   __shared__ float s_part[4][kRouteTokens][8];
   const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kRouteTokens;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.num_experts;
+  const bool softmax_chosen = a.score_mode == HYMETA_ROUTE_SOFTMAX_CHOSEN;
   const int live = min(static_cast<int64_t>(kRouteTokens), a.num_tokens - t0);
   const elem* x[kRouteTokens];
 #pragma unroll
@@ -51,7 +52,10 @@ __global__ __launch_bounds__(256) void moe_scores_topk_kernel(hymeta_moe_route_s
     __syncthreads();
     if (threadIdx.x < kRouteTokens * 8) {
       const int i = threadIdx.x >> 3, j = threadIdx.x & 7;
-      if (e0 + j < E) s_score[i][e0 + j] = sigmoid_exact((s_part[0][i][j] + s_part[1][i][j]) + (s_part[2][i][j] + s_part[3][i][j]));
+      if (e0 + j < E) {
+        const float z = (s_part[0][i][j] + s_part[1][i][j]) + (s_part[2][i][j] + s_part[3][i][j]) + (a.router_bias ? a.router_bias[e0 + j] : 0.f);
+        s_score[i][e0 + j] = softmax_chosen ? z : sigmoid_exact(z);
+      }
     }
     __syncthreads();
   }
@@ -60,7 +64,7 @@ __global__ __launch_bounds__(256) void moe_scores_topk_kernel(hymeta_moe_route_s
   float* score = s_score[wave];
   float total = 0.f;
   for (int k = 0; k < a.top_k; ++k) {
-    float best = -2.f;
+    float best = -INFINITY;
     int arg = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
       const float v = score[e];
@@ -74,10 +78,18 @@ __global__ __launch_bounds__(256) void moe_scores_topk_kernel(hymeta_moe_route_s
     if (lane == 0) {
       a.topk_ids[t * a.top_k + k] = cand;
       s_top[wave][k] = top;
-      score[cand] = -1.f;                         // scores are >= 0: taken
+      score[cand] = -INFINITY;                    // taken
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
+  }
+  if (softmax_chosen) {
+    // the first chosen logit is the largest: exponentials of the differences to it, over their sum
+    const float top0 = s_top[wave][0];
+    float sum = 0.f;
+    for (int k = 0; k < a.top_k; ++k) sum += expf(s_top[wave][k] - top0);
+    for (int k = lane; k < a.top_k; k += 64) a.topk_weights[t * a.top_k + k] = expf(s_top[wave][k] - top0) / sum * a.scale;
+    return;
   }
   const float inv = a.scale / (total + 1e-20f);
   for (int k = lane; k < a.top_k; k += 64) a.topk_weights[t * a.top_k + k] = s_top[wave][k] * inv;
@@ -125,6 +137,7 @@ extern "C" int hymeta_moe_route_sigmoid(const hymeta_moe_route_sigmoid_args* arg
   if (a.num_tokens < 0 || a.num_experts <= 0 || a.top_k <= 0 || a.hidden <= 0) return HYMETA_ERR_INVALID_ARG;
   if (a.num_experts > HYMETA_MOE_TABLE_MAX_EXPERTS || a.top_k > a.num_experts) return HYMETA_ERR_UNSUPPORTED;
   if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
+  if (a.score_mode != HYMETA_ROUTE_SIGMOID_SUM && a.score_mode != HYMETA_ROUTE_SOFTMAX_CHOSEN) return HYMETA_ERR_UNSUPPORTED;
   if (!a.expert_offsets) return HYMETA_ERR_INVALID_ARG;
   if (a.num_tokens > 0 && (!a.x || !a.router_weight || !a.topk_ids || !a.topk_weights || !a.sorted_pair || !a.pair_pos || a.x_stride_t < a.hidden))
     return HYMETA_ERR_INVALID_ARG;

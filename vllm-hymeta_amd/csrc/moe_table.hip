@@ -137,6 +137,10 @@ __global__ __launch_bounds__(256) void moe_gemm_any_kernel(hymeta_moe_gemm_any_a
           v = gte * sigmoid_exact(gte) * up;
         }
       }
+      if (!Gated && a.gated == HYMETA_GLU_RELU2) {
+        const float r = fmaxf(A::round(v), 0.f);       // the projection's output as a GEMM would store it
+        v = r * r;
+      }
       A::st(orow + n, v * sc);
     }
   }
@@ -180,7 +184,7 @@ extern "C" int hymeta_moe_gemm_any(const hymeta_moe_gemm_any_args* args, hymeta_
   const hymeta_moe_gemm_any_args& a = *args;
   if (a.max_rows < 0 || a.K <= 0 || a.N <= 0 || a.num_experts <= 0) return HYMETA_ERR_INVALID_ARG;
   if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
-  if (a.gated != HYMETA_GLU_NONE && a.gated != HYMETA_GLU_SILU && a.gated != HYMETA_GLU_CLAMPED) return HYMETA_ERR_UNSUPPORTED;
+  if (a.gated < HYMETA_GLU_NONE || a.gated > HYMETA_GLU_RELU2) return HYMETA_ERR_UNSUPPORTED;
   if (a.max_rows == 0) return HYMETA_OK;
   if (!a.x || !a.weights || !a.out || !a.expert_offsets) return HYMETA_ERR_INVALID_ARG;
   if (a.a_rows != nullptr && a.a_rows_div <= 0) return HYMETA_ERR_INVALID_ARG;
@@ -190,7 +194,7 @@ extern "C" int hymeta_moe_gemm_any(const hymeta_moe_gemm_any_args* args, hymeta_
   const dim3 grid((a.N + kBN - 1) / kBN, static_cast<unsigned>(tiles));
   hipStream_t st = begin_launches(stream);
   const bool bf = a.act_dtype == HYMETA_BF16;
-  if (a.gated) {
+  if (a.gated == HYMETA_GLU_SILU || a.gated == HYMETA_GLU_CLAMPED) {
     if (bf) hipLaunchKernelGGL((moe_gemm_any_kernel<ActBf16, true>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((moe_gemm_any_kernel<ActF32, true>), grid, dim3(256), 0, st, a);
   } else {

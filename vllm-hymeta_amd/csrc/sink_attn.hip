@@ -10,7 +10,7 @@ namespace hymeta {
 
 namespace {
 
-constexpr int kMaxHeadDim = 1024;
+constexpr int kMaxHeadDim = 4096;
 constexpr int kMaxVChunks = 8;       // value size <= 512
 
 // grid = tokens; a wave per (token, head) task: query heads, then key heads, then value heads.
@@ -79,47 +79,54 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
   for (int d = lane; d < D; d += 64) s_q[d] = A::ld(q + d);
   const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
   const elem* cache = static_cast<const elem*>(a.kv_cache);
-  // a head's part of a cache row: its key followed by its value, or a key whose first Dv elements are the value
-  const int head_elems = a.kv_layout == HYMETA_KV_VALUE_IN_KEY ? D : D + Dv;
-  const int v_off = a.kv_layout == HYMETA_KV_VALUE_IN_KEY ? 0 : D;
-  const int64_t row_elems = static_cast<int64_t>(G) * head_elems;
+  // where the head's key and value lie in a cache row: a key followed by its value per key/value head; a key whose first Dv
+  // elements are the value; or one key for all heads followed by the key/value heads' values
+  int64_t row_elems, key_off, val_off;
+  if (a.kv_layout == HYMETA_KV_SHARED_KEY) row_elems = D + static_cast<int64_t>(G) * Dv, key_off = 0, val_off = D + static_cast<int64_t>(g) * Dv;
+  else if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY) row_elems = static_cast<int64_t>(G) * D, key_off = static_cast<int64_t>(g) * D, val_off = key_off;
+  else row_elems = static_cast<int64_t>(G) * (D + Dv), key_off = static_cast<int64_t>(g) * (D + Dv), val_off = key_off + D;
   const float ba = a.bias_mode ? a.bias_a[h] : 0.f, bb = a.bias_mode ? a.bias_b[h] : 0.f;
   // the sink: a key of score sink_logits[h] (0 without) that has no value
   float m = a.sink ? (a.sink_logits ? a.sink_logits[h] : 0.f) : -INFINITY, l = a.sink ? 1.f : 0.f;
   float acc[kMaxVChunks] = {};
   const int nvc = (Dv + 63) / 64;
   __syncthreads();
-  for (int j0 = first; j0 <= pos; j0 += 64) {
-    const int j = j0 + lane;
-    const bool valid = j <= pos;
-    float sc = -INFINITY;
-    int64_t roff = 0;
-    if (valid) {
-      const int64_t blk = bt[j / a.block_size];
-      roff = (blk * a.block_size + j % a.block_size) * row_elems + static_cast<int64_t>(g) * head_elems;
-      const elem* k = cache + roff;
-      float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot = fmaf(s_q[d], A::ld(k + d), dot);
-      sc = dot * a.scale - distance_bias(a.bias_mode, ba, bb, pos - j);
-    }
-    const float m_new = fmaxf(m, wave_max(sc));
-    const float p = valid ? expf(sc - m_new) : 0.f;
-    const float corr = expf(m - m_new);            // m = -inf only without a sink before the first tile: corr = 0, l = 0
-    l = l * corr + wave_sum(p);
-    m = m_new;
-    __syncthreads();
-    s_p[lane] = p;
-    s_row[lane] = roff + v_off;
-    __syncthreads();
-    const int n = min(64, pos - j0 + 1);
+  // two runs of keys: the kept first ones that lie before the window, then the window
+  const int kept = a.window_left >= 0 ? min(a.keep_first, first) : 0;
+  for (int run = 0; run < 2; ++run) {
+    const int lo = run == 0 ? 0 : first, hi = run == 0 ? kept - 1 : pos;
+    for (int j0 = lo; j0 <= hi; j0 += 64) {
+      const int j = j0 + lane;
+      const bool valid = j <= hi;
+      float sc = -INFINITY;
+      int64_t roff = 0;
+      if (valid) {
+        const int64_t blk = bt[j / a.block_size];
+        roff = (blk * a.block_size + j % a.block_size) * row_elems;
+        const elem* k = cache + roff + key_off;
+        float dot = 0.f;
+        for (int d = 0; d < D; ++d) dot = fmaf(s_q[d], A::ld(k + d), dot);
+        sc = dot * a.scale - distance_bias(a.bias_mode, ba, bb, pos - j);
+      }
+      const float m_new = fmaxf(m, wave_max(sc));
+      const float p = valid ? expf(sc - m_new) : 0.f;
+      const float corr = expf(m - m_new);            // m = -inf only without a sink before the first tile: corr = 0, l = 0
+      l = l * corr + wave_sum(p);
+      m = m_new;
+      __syncthreads();
+      s_p[lane] = p;
+      s_row[lane] = roff + val_off;
+      __syncthreads();
+      const int n = min(64, hi - j0 + 1);
 #pragma unroll
-    for (int cc = 0; cc < kMaxVChunks; ++cc) {
-      if (cc < nvc) {
-        const int c = cc * 64 + lane;
-        float r = acc[cc] * corr;
-        if (c < Dv)
-          for (int jj = 0; jj < n; ++jj) r = fmaf(s_p[jj], A::ld(cache + s_row[jj] + c), r);
-        acc[cc] = r;
+      for (int cc = 0; cc < kMaxVChunks; ++cc) {
+        if (cc < nvc) {
+          const int c = cc * 64 + lane;
+          float r = acc[cc] * corr;
+          if (c < Dv)
+            for (int jj = 0; jj < n; ++jj) r = fmaf(s_p[jj], A::ld(cache + s_row[jj] + c), r);
+          acc[cc] = r;
+        }
       }
     }
   }
@@ -687,6 +694,7 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
 // over value slices of 128 (each repeats the scores over the whole key: 1.5 to 2.1 times the matrix work of one pass
 // with accumulators for all the value columns, which do not fit a wave's registers beside the query fragments).
 inline bool mfma_shape(const hymeta_sink_attention_args& a) {
+  if (a.kv_layout == HYMETA_KV_SHARED_KEY || (a.window_left >= 0 && a.keep_first > 0)) return false;
   bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
   if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY)
     dims = ((a.v_dim == 64 || a.v_dim == 128) && (a.head_dim == a.v_dim + 32 || a.head_dim == a.v_dim + 64)) ||
@@ -778,7 +786,8 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
   if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
   if (a.head_dim > kMaxHeadDim || a.v_dim > 64 * kMaxVChunks) return HYMETA_ERR_UNSUPPORTED;
   if (a.bias_mode != HYMETA_BIAS_NONE && a.bias_mode != HYMETA_BIAS_LOG_DISTANCE) return HYMETA_ERR_UNSUPPORTED;
-  if (a.kv_layout != HYMETA_KV_KEY_THEN_VALUE && a.kv_layout != HYMETA_KV_VALUE_IN_KEY) return HYMETA_ERR_UNSUPPORTED;
+  if (a.kv_layout != HYMETA_KV_KEY_THEN_VALUE && a.kv_layout != HYMETA_KV_VALUE_IN_KEY && a.kv_layout != HYMETA_KV_SHARED_KEY) return HYMETA_ERR_UNSUPPORTED;
+  if (a.window_left >= 0 && a.keep_first < 0) return HYMETA_ERR_INVALID_ARG;
   if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY && a.v_dim > a.head_dim) return HYMETA_ERR_INVALID_ARG;
   if (a.num_tokens == 0 || a.num_seqs == 0) return HYMETA_OK;
   if (!a.q || !a.kv_cache || !a.out || !a.block_tables || !a.query_start_loc || !a.seq_lens) return HYMETA_ERR_INVALID_ARG;

@@ -28,12 +28,15 @@ BIAS_NONE = 0
 BIAS_LOG_DISTANCE = 1
 KV_KEY_THEN_VALUE = 0
 KV_VALUE_IN_KEY = 1
-GLU_NONE, GLU_SILU, GLU_CLAMPED = 0, 1, 2
-ACT_CLAMPED_GLU, ACT_XIELU, ACT_SIGMOID_MUL = 0, 1, 2
+KV_SHARED_KEY = 2
+GLU_NONE, GLU_SILU, GLU_CLAMPED, GLU_RELU2 = 0, 1, 2, 3
+ACT_CLAMPED_GLU, ACT_XIELU, ACT_SIGMOID_MUL, ACT_SILU_MUL, ACT_RELU2 = 0, 1, 2, 3, 4
+ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN = 0, 1
+MAX_STREAMS = 8
 LIGHTNING_CHUNK = 64
 CONV_MAX_TAPS = 8
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 ERR_SCRATCH_LIMIT = -5
 GEMM_TICKET_BYTES = 16384
 STATIC_SCRATCH_BYTES = 16 << 20
@@ -356,7 +359,7 @@ class SinkAttentionArgs(_Args):
         ("bias_mode", _i32), ("sink", _i32), ("window_left", _i32), ("max_query_len", _i32), ("max_seq_len", _i32),
         ("scale", _f32),
         ("num_blocks", _i64), ("q_stride_t", _i64), ("block_table_stride", _i64),
-        ("sink_logits", _ptr), ("kv_layout", _i32),
+        ("sink_logits", _ptr), ("kv_layout", _i32), ("keep_first", _i32),
     ]
 
 
@@ -472,6 +475,40 @@ class MoeRouteSigmoidArgs(_Args):
         ("num_tokens", _i32), ("num_experts", _i32), ("top_k", _i32), ("hidden", _i32), ("act_dtype", _i32),
         ("scale", _f32),
         ("x_stride_t", _i64),
+        ("router_bias", _ptr), ("score_mode", _i32),
+    ]
+
+
+class EmbedPairArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("token_ids", _ptr), ("table", _ptr), ("pair_table", _ptr), ("norm_weight", _ptr), ("out", _ptr), ("prev_token", _ptr),
+        ("first_rows", _ptr), ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("width", _i32), ("vocab", _i32), ("copies", _i32), ("act_dtype", _i32),
+        ("buckets", _i64), ("mul_prev", _i64), ("mul_cur", _i64),
+        ("eps", _f32),
+    ]
+
+
+class HyperStreamArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("y", _ptr), ("mix", _ptr), ("out_w", _ptr), ("in_w", _ptr), ("norm_weight", _ptr), ("h_out", _ptr),
+        ("num_tokens", _i32), ("streams", _i32), ("width", _i32), ("act_dtype", _i32),
+        ("eps", _f32),
+        ("y_stride_t", _i64),
+    ]
+
+
+class TalkQkvPrepArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("qkv", _ptr), ("q_weight", _ptr), ("k_weight", _ptr), ("talk", _ptr), ("rot_freqs", _ptr), ("v_other", _ptr), ("q_out", _ptr),
+        ("kv_cache", _ptr), ("slot_mapping", _ptr), ("query_start_loc", _ptr), ("seq_lens", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32), ("v_dim", _i32),
+        ("rot_dims", _i32), ("block_size", _i32), ("act_dtype", _i32),
+        ("eps", _f32), ("v_blend", _f32),
+        ("num_blocks", _i64), ("qkv_stride_t", _i64), ("v_other_stride_t", _i64),
     ]
 
 
@@ -562,6 +599,9 @@ _SIGNATURES = {
     "hymeta_gated_rms_norm": (C.c_int, [C.POINTER(GatedRmsNormArgs), _ptr]),
     "hymeta_activation": (C.c_int, [C.POINTER(ActivationArgs), _ptr]),
     "hymeta_moe_route_sigmoid": (C.c_int, [C.POINTER(MoeRouteSigmoidArgs), _ptr]),
+    "hymeta_embed_pair": (C.c_int, [C.POINTER(EmbedPairArgs), _ptr]),
+    "hymeta_hyper_stream": (C.c_int, [C.POINTER(HyperStreamArgs), _ptr]),
+    "hymeta_talk_qkv_prep": (C.c_int, [C.POINTER(TalkQkvPrepArgs), _ptr]),
 }
 
 STRUCTS = {
@@ -600,6 +640,9 @@ STRUCTS = {
     "hymeta_gated_rms_norm_args": GatedRmsNormArgs,
     "hymeta_activation_args": ActivationArgs,
     "hymeta_moe_route_sigmoid_args": MoeRouteSigmoidArgs,
+    "hymeta_embed_pair_args": EmbedPairArgs,
+    "hymeta_hyper_stream_args": HyperStreamArgs,
+    "hymeta_talk_qkv_prep_args": TalkQkvPrepArgs,
 }
 
 

@@ -1600,7 +1600,8 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
                    seq_lens: torch.Tensor, num_kv_heads: int, head_dim: int, v_dim: int, scale: float,
                    max_query_len: int, max_seq_len: int, bias_a: Optional[torch.Tensor] = None,
                    bias_b: Optional[torch.Tensor] = None, sink: bool = True, window_left: int = -1,
-                   sink_logits: Optional[torch.Tensor] = None, value_in_key: bool = False) -> torch.Tensor:
+                   sink_logits: Optional[torch.Tensor] = None, value_in_key: bool = False, shared_key: bool = False,
+                   keep_first: int = 0) -> torch.Tensor:
     """Causal attention of the rows ``q [T, H, D]`` over their sequences' paged keys (this step's included):
     ``softmax`` over ``scale q.k - bias_a[h] ln(1 + bias_b[h] (i - j))`` with, for ``sink``, ``exp(sink_logits[h])`` (one
     without ``sink_logits``) added to the denominator.  ``value_in_key``: a cache row holds ``D`` elements per key/value
@@ -1610,8 +1611,11 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
     T, H, _ = q.shape
     row = head_dim if value_in_key else head_dim + v_dim
     _require(not value_in_key or v_dim <= head_dim, "a value inside its key cannot be longer than the key")
+    _require(not (value_in_key and shared_key), "one row layout at a time")
+    cache_tail = (1, head_dim + num_kv_heads * v_dim) if shared_key else (num_kv_heads, row)
     _require(kv_cache.dtype == q.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4
-             and kv_cache.shape[2:] == (num_kv_heads, row), f"kv_cache must be contiguous [blocks, block_size, G, {row}]")
+             and kv_cache.shape[2:] == cache_tail, f"kv_cache must be contiguous [blocks, block_size, {cache_tail[0]}, {cache_tail[1]}]")
+    _require(keep_first >= 0, "keep_first counts tokens")
     _f32vec(sink_logits, H, "sink_logits")
     S = query_start_loc.numel() - 1
     _i32vec(query_start_loc, S + 1, "query_start_loc")
@@ -1634,7 +1638,8 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
     a.block_size, a.act_dtype, a.num_blocks = kv_cache.shape[1], _act(q), kv_cache.shape[0]
     a.bias_mode = _C.BIAS_NONE if bias_a is None else _C.BIAS_LOG_DISTANCE
     a.sink, a.window_left, a.max_query_len, a.max_seq_len, a.scale = int(bool(sink)), window_left, max_query_len, max_seq_len, scale
-    a.sink_logits, a.kv_layout = _p(sink_logits), (_C.KV_VALUE_IN_KEY if value_in_key else _C.KV_KEY_THEN_VALUE)
+    a.sink_logits, a.keep_first = _p(sink_logits), keep_first
+    a.kv_layout = _C.KV_SHARED_KEY if shared_key else (_C.KV_VALUE_IN_KEY if value_in_key else _C.KV_KEY_THEN_VALUE)
     a.q_stride_t, a.block_table_stride = q.stride(0), block_tables.stride(0)
     _C.check(lib.hymeta_sink_attention(C.byref(a), _stream(q)), "hymeta_sink_attention")
     return out
@@ -1916,21 +1921,40 @@ def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
     return _activation(_C.ACT_SIGMOID_MUL, x, x.shape[1], 0.0, 0.0, gate=gate)
 
 
+ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN = _C.ROUTE_SIGMOID_SUM, _C.ROUTE_SOFTMAX_CHOSEN
+
+
 def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, top_k: int,
                         route_scale: float, limit: float, alpha: float = 1.702) -> torch.Tensor:
     """Experts chosen by the ``top_k`` largest ``sigmoid(x router_weight^T)`` (fp32), weighing their scores over the
     chosen's sum times ``route_scale``; every expert is a clamped gated unit (``clamped_glu``) between ``w13 [E, 2I, H]``
     (gate rows, then up rows) and ``w2 [E, H, I]``, all bf16 or all fp32.  bf16 experts in the MFMA tiles' shapes run the
     routed block's grouped GEMMs, everything else the generic grouped GEMM with the activation in its epilogue."""
-    _dev(x, router_weight, w13, w2)
+    return moe_routed_forward(x, router_weight, None, w13, w2, top_k, _C.ROUTE_SIGMOID_SUM, route_scale, "clamped_glu", limit, alpha)
+
+
+def moe_routed_forward(x: torch.Tensor, router_weight: torch.Tensor, router_bias: Optional[torch.Tensor], w1: torch.Tensor,
+                       w2: torch.Tensor, top_k: int, score_mode: int, route_scale: float, expert_act: str, limit: float = 0.0,
+                       alpha: float = 1.702) -> torch.Tensor:
+    """Experts chosen by the ``top_k`` largest router logits ``x router_weight^T (+ router_bias)`` (fp32; the lower expert
+    on a tie).  ``score_mode``: ``ROUTE_SIGMOID_SUM`` (weights = sigmoid scores over the chosen's sum) or
+    ``ROUTE_SOFTMAX_CHOSEN`` (softmax over the chosen logits alone), times ``route_scale``.  ``expert_act``:
+    ``"clamped_glu"``: ``w1 [E, 2I, H]`` (gate rows, then up rows), ``g sigmoid(alpha g) (u + 1)`` clamped at ``limit``;
+    ``"relu2"``: ``w1 [E, I, H]``, ``max(z, 0)^2``.  ``w2 [E, H, I]``; all bf16 or all fp32.  bf16 experts in the MFMA
+    tiles' shapes run the routed block's grouped GEMMs, everything else the generic grouped GEMM with the activation in its
+    epilogue."""
+    _dev(x, router_weight, router_bias, w1, w2)
+    _require(expert_act in ("clamped_glu", "relu2"), "expert_act is clamped_glu or relu2")
+    gated = expert_act == "clamped_glu"
     T, H = x.shape
-    E, two_i, _ = w13.shape
-    inter = two_i // 2
-    _require(x.dtype in _DT and x.stride(1) == 1 and w13.dtype == x.dtype and w2.dtype == x.dtype, "x, w13 and w2 must share bf16 or fp32")
-    _require(w13.is_contiguous() and w13.shape == (E, 2 * inter, H) and w2.is_contiguous() and w2.shape == (E, H, inter),
-             "w13 must be contiguous [E, 2I, H] and w2 [E, H, I]")
+    E, n1, _ = w1.shape
+    inter = n1 // 2 if gated else n1
+    _require(x.dtype in _DT and x.stride(1) == 1 and w1.dtype == x.dtype and w2.dtype == x.dtype, "x, w1 and w2 must share bf16 or fp32")
+    _require(w1.is_contiguous() and w1.shape == (E, (2 if gated else 1) * inter, H) and w2.is_contiguous() and w2.shape == (E, H, inter),
+             "w1 must be contiguous [E, 2I or I, H] and w2 [E, H, I]")
     _require(router_weight.dtype == torch.float32 and router_weight.is_contiguous() and router_weight.shape == (E, H),
              "router_weight must be contiguous fp32 [E, H]")
+    _f32vec(router_bias, E, "router_bias")
     dev = x.device
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     if T == 0:
@@ -1946,17 +1970,18 @@ def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch
     r.x, r.router_weight, r.topk_ids, r.topk_weights = _p(x), _p(router_weight), _p(ids), _p(wts)
     r.expert_offsets, r.sorted_pair, r.pair_pos = _p(offsets), _p(sorted_pair), _p(pair_pos)
     r.num_tokens, r.num_experts, r.top_k, r.hidden, r.act_dtype, r.scale, r.x_stride_t = T, E, top_k, H, _act(x), route_scale, x.stride(0)
+    r.router_bias, r.score_mode = _p(router_bias), score_mode
     _C.check(lib.hymeta_moe_route_sigmoid(C.byref(r), st), "hymeta_moe_route_sigmoid")
 
-    if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and E <= 64 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
-        h13 = torch.empty(P, two_i, dtype=torch.bfloat16, device=dev)
+    if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and n1 % 64 == 0 and E <= 64 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+        h1 = torch.empty(P, n1, dtype=torch.bfloat16, device=dev)
         g = _C.MoeGemmArgs()
-        g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(h13), _p(offsets)
-        g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N = _p(sorted_pair), top_k, P, H, two_i
+        g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w1), _p(h1), _p(offsets)
+        g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N = _p(sorted_pair), top_k, P, H, n1
         g.local_expert_begin, g.local_expert_end = 0, E
-        g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), h13.stride(0), w13.stride(0)
-        _C.check(lib.hymeta_moe_gemm(C.byref(g), st), "hymeta_moe_gemm (w13)")
-        hact = clamped_glu(h13, limit, alpha)
+        g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), h1.stride(0), w1.stride(0)
+        _C.check(lib.hymeta_moe_gemm(C.byref(g), st), "hymeta_moe_gemm (w1)")
+        hact = clamped_glu(h1, limit, alpha) if gated else relu_squared(h1, out=h1)
         y = torch.empty(P, H, dtype=torch.bfloat16, device=dev)
         d = _C.MoeGemmArgs()
         d.x, d.x_stride_m, d.weights, d.out, d.expert_offsets = _p(hact), hact.stride(0), _p(w2), _p(y), _p(offsets)
@@ -1975,11 +2000,12 @@ def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch
     act = _DT[x.dtype]
     hact = torch.empty(P, inter, dtype=x.dtype, device=dev)
     g = _C.MoeGemmAnyArgs()
-    g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(hact), _p(offsets)
-    g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N, g.num_experts, g.gated, g.act_dtype = _p(sorted_pair), top_k, P, H, inter, E, _C.GLU_CLAMPED, act
+    g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w1), _p(hact), _p(offsets)
+    g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N, g.num_experts, g.act_dtype = _p(sorted_pair), top_k, P, H, inter, E, act
+    g.gated = _C.GLU_CLAMPED if gated else _C.GLU_RELU2
     g.act_limit, g.act_alpha = limit, alpha
-    g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), hact.stride(0), w13.stride(0)
-    _C.check(lib.hymeta_moe_gemm_any(C.byref(g), st), "hymeta_moe_gemm_any (w13)")
+    g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), hact.stride(0), w1.stride(0)
+    _C.check(lib.hymeta_moe_gemm_any(C.byref(g), st), "hymeta_moe_gemm_any (w1)")
     y = torch.empty(P, H, dtype=x.dtype, device=dev)
     d = _C.MoeGemmAnyArgs()
     d.x, d.weights, d.out, d.expert_offsets = _p(hact), _p(w2), _p(y), _p(offsets)
@@ -1993,3 +2019,121 @@ def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch
     c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
     _C.check(lib.hymeta_moe_combine_any(C.byref(c), st), "hymeta_moe_combine_any")
     return out
+
+
+def silu_mul(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x [rows, 2 n]`` (gate columns, then up columns) -> ``gate sigmoid(gate) up``, bf16 or fp32 (``silu_and_mul`` is the
+    bf16-only form of the quantised linears' path)."""
+    _require(x.shape[1] % 2 == 0, "x must hold the gate and the up columns")
+    return _activation(_C.ACT_SILU_MUL, x, x.shape[1] // 2, 0.0, 0.0, out=out)
+
+
+def relu_squared(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``max(x, 0)^2`` (``out`` may be ``x``)."""
+    return _activation(_C.ACT_RELU2, x, x.shape[1], 0.0, 0.0, out=out)
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of pre-norm designs with several residual streams and head-mixed attention scores.
+# ---------------------------------------------------------------------------
+def embed_pair(token_ids: torch.Tensor, table: torch.Tensor, pair_table: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor],
+               eps: float, copies: int, buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0, prev_token: Optional[torch.Tensor] = None,
+               query_start_loc: Optional[torch.Tensor] = None, context_lens: Optional[torch.Tensor] = None,
+               slot_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 ``[T, copies, W]``: ``layer_norm(table[token] + pair_table[row]) * norm_weight`` in every copy, with ``row =
+    (previous token * mul_prev + token * mul_cur) mod buckets`` and row ``buckets`` for a sequence's first token.
+    ``prev_token`` int32 ``[slots]`` carries every sequence's last token between steps and is updated in place."""
+    _dev(token_ids, table, pair_table, norm_weight, prev_token, query_start_loc, context_lens, slot_idx)
+    _require(token_ids.dtype == torch.int64 and token_ids.dim() == 1 and token_ids.is_contiguous(), "token_ids must be contiguous int64 [T]")
+    _require(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [vocab, width]")
+    V, W = table.shape
+    T = token_ids.shape[0]
+    _f32vec(norm_weight, W, "norm_weight")
+    out = torch.empty(T, copies, W, dtype=torch.float32, device=table.device)
+    a = _C.EmbedPairArgs()
+    a.token_ids, a.table, a.norm_weight, a.out = _p(token_ids), _p(table), _p(norm_weight), _p(out)
+    a.num_tokens, a.width, a.vocab, a.copies, a.act_dtype, a.eps = T, W, V, copies, _act(table), eps
+    if pair_table is not None:
+        _require(pair_table.dtype == table.dtype and pair_table.is_contiguous() and pair_table.shape == (buckets + 1, W),
+                 "pair_table must be contiguous [buckets + 1, width] of the table's type")
+        S = query_start_loc.numel() - 1
+        _i32vec(query_start_loc, S + 1, "query_start_loc")
+        _i32vec(context_lens, S, "context_lens")
+        _i32vec(slot_idx, S, "slot_idx")
+        _require(prev_token is not None and prev_token.dtype == torch.int32 and prev_token.is_contiguous(), "prev_token must be contiguous int32 [slots]")
+        first_rows = torch.empty(max(S, 1), dtype=torch.int32, device=table.device)
+        a.pair_table, a.prev_token, a.first_rows = _p(pair_table), _p(prev_token), _p(first_rows)
+        a.query_start_loc, a.context_lens, a.slot_idx, a.num_seqs = _p(query_start_loc), _p(context_lens), _p(slot_idx), S
+        a.buckets, a.mul_prev, a.mul_cur = buckets, mul_prev, mul_cur
+    _C.check(_C.load().hymeta_embed_pair(C.byref(a), _stream(table)), "hymeta_embed_pair")
+    return out
+
+
+def hyper_stream_(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torch.Tensor], out_w: Optional[torch.Tensor],
+                  in_w: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor], eps: float,
+                  h_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+    """One step of the residual streams ``x [T, S, W]`` fp32, in place: with ``y [T, W]``, ``x_t <- sum_s mix[s, t] x_s +
+    out_w[t] y``; with ``h_dtype``, returns ``layer_norm(sum_s in_w[s] x_s) * norm_weight`` of the new streams in that
+    type (``norm_weight`` None: the weighted sum itself)."""
+    _dev(x, y, mix, out_w, in_w, norm_weight)
+    _require(x.dtype == torch.float32 and x.dim() == 3 and x.is_contiguous(), "x must be contiguous fp32 [T, S, W]")
+    T, S, W = x.shape
+    _require(y is not None or h_dtype is not None, "nothing to do")
+    a = _C.HyperStreamArgs()
+    a.x, a.num_tokens, a.streams, a.width, a.eps = _p(x), T, S, W, eps
+    act = h_dtype
+    if y is not None:
+        _require(y.dim() == 2 and y.shape == (T, W) and y.stride(1) == 1 and y.dtype in _DT, "y must be row-contiguous [T, W]")
+        _f32vec(mix, S * S, "mix")
+        _f32vec(out_w, S, "out_w")
+        _require(h_dtype is None or h_dtype == y.dtype, "the sublayer's output and the next input share a type")
+        a.y, a.mix, a.out_w, a.y_stride_t = _p(y), _p(mix), _p(out_w), y.stride(0)
+        act = y.dtype
+    h = None
+    if h_dtype is not None:
+        _f32vec(in_w, S, "in_w")
+        _f32vec(norm_weight, W, "norm_weight")
+        h = torch.empty(T, W, dtype=h_dtype, device=x.device)
+        a.in_w, a.norm_weight, a.h_out = _p(in_w), _p(norm_weight), _p(h)
+    a.act_dtype = _DT[act]
+    _C.check(_C.load().hymeta_hyper_stream(C.byref(a), _stream(x)), "hymeta_hyper_stream")
+    return h
+
+
+def talk_qkv_prep(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int, q_weight: torch.Tensor,
+                  k_weight: torch.Tensor, talk: torch.Tensor, eps: float, rot_dims: int, rot_freqs: Optional[torch.Tensor],
+                  kv_cache: torch.Tensor, slot_mapping: torch.Tensor, query_start_loc: torch.Tensor, seq_lens: torch.Tensor,
+                  v_other: Optional[torch.Tensor] = None, v_blend: float = 0.0) -> torch.Tensor:
+    """From ``qkv [T, H D + G D + G Dv]``: RMS norms over the whole query and key projections, rotation of the first
+    ``rot_dims`` dimensions of every head in interleaved pairs, values blended with ``v_other`` (``(1 - v_blend) v + v_blend
+    v_other``), the paged write of ``(keys of all G heads, values of all G heads)`` into ``kv_cache [blocks, block_size, 1,
+    G D + G Dv]``; returns the queries mixed across heads, ``[T, H, G D]``: ``out[h, g D + d] = sum_j talk[h, j] q[j, d]``
+    over the query heads ``j`` of group ``g``."""
+    _dev(qkv, q_weight, k_weight, talk, rot_freqs, kv_cache, slot_mapping, query_start_loc, seq_lens, v_other)
+    T = qkv.shape[0]
+    H, G, D, Dv = num_heads, num_kv_heads, head_dim, v_dim
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (H + G) * D + G * Dv and qkv.dtype in _DT,
+             "qkv must be row-contiguous [T, H D + G D + G Dv]")
+    _f32vec(q_weight, H * D, "q_weight")
+    _f32vec(k_weight, G * D, "k_weight")
+    _f32vec(talk, H * H, "talk")
+    _require(rot_dims == 0 or (rot_freqs is not None and rot_freqs.dtype == torch.float64 and rot_freqs.is_contiguous()
+                               and rot_freqs.numel() == rot_dims // 2), "rot_freqs must be contiguous float64 [rot_dims / 2]")
+    _require(kv_cache.dtype == qkv.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4 and kv_cache.shape[2:] == (1, G * (D + Dv)),
+             "kv_cache must be contiguous [blocks, block_size, 1, G D + G Dv]")
+    _require(slot_mapping.dtype == torch.int64 and slot_mapping.is_contiguous() and slot_mapping.numel() == T, "slot_mapping must be int64 [T]")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(seq_lens, S, "seq_lens")
+    q_out = torch.empty(T, H, G * D, dtype=qkv.dtype, device=qkv.device)
+    a = _C.TalkQkvPrepArgs()
+    a.qkv, a.q_weight, a.k_weight, a.talk, a.rot_freqs, a.q_out = _p(qkv), _p(q_weight), _p(k_weight), _p(talk), _p(rot_freqs), _p(q_out)
+    a.kv_cache, a.slot_mapping, a.query_start_loc, a.seq_lens = _p(kv_cache), _p(slot_mapping), _p(query_start_loc), _p(seq_lens)
+    a.num_tokens, a.num_seqs, a.num_heads, a.num_kv_heads, a.head_dim, a.v_dim, a.rot_dims = T, S, H, G, D, Dv, rot_dims
+    a.block_size, a.num_blocks, a.act_dtype, a.eps, a.qkv_stride_t = kv_cache.shape[1], kv_cache.shape[0], _act(qkv), eps, qkv.stride(0)
+    if v_other is not None:
+        _require(v_other.dim() == 2 and v_other.shape == (T, G * Dv) and v_other.stride(1) == 1 and v_other.dtype == qkv.dtype,
+                 "v_other must be row-contiguous [T, G Dv] of qkv's type")
+        a.v_other, a.v_other_stride_t, a.v_blend = _p(v_other), v_other.stride(0), v_blend
+    _C.check(_C.load().hymeta_talk_qkv_prep(C.byref(a), _stream(qkv)), "hymeta_talk_qkv_prep")
+    return q_out

@@ -1,10 +1,13 @@
-"""Feed-forward sublayers of the post-norm designs:
+"""Feed-forward sublayers of the designs on fp32 residual streams:
 
 ``XieluMLP``        ``W_down xielu(W_up h + b_up) + b_down`` with ``xielu(z) = a_pos z^2 + z / 2`` for ``z > 0`` and
                     ``a_neg (exp(z) - 1 - z) + z / 2`` otherwise, ``a_pos = softplus(p)``, ``a_neg = 1/2 + softplus(q)``
 ``ClampedGluMLP``   ``W_down (g sigmoid(alpha g) (u + 1))`` with ``g = min(W_gate h, limit)``, ``u = clamp(W_up h, +-limit)``
 ``SigmoidRoutedMoE``  experts of the second form chosen by the largest ``sigmoid`` router scores, weighing their scores
                     over the chosen's sum times a constant, beside an optional shared expert that every token runs
+``SiluGluMLP``      ``W_down (silu(W_gate h + b_gate) (W_up h + b_up)) + b_down``, bf16 or fp32
+``Relu2RoutedMoE``  experts ``W_down max(W_up h, 0)^2`` chosen by the largest router logits ``W_r h + b_r``, weighing the
+                    softmax over the chosen logits alone
 
 Beside ``HymetaMoE`` (``moe.py``: softmax router, silu experts) and ``TableMoE`` (``table_moe.py``: no router network);
 the expert stacks ``w13 [E, 2I, H]`` / ``w2 [E, H, I]`` are theirs.
@@ -60,3 +63,28 @@ class SigmoidRoutedMoE(torch.nn.Module):
         """``(routed experts' weighted sum, shared expert's output or None)``: whoever adds them to the stream adds both."""
         y = hip_ops.moe_sigmoid_forward(h, self.router_weight, self.w13, self.w2, self.top_k, self.route_scale, self.limit, self.alpha)
         return y, (None if self.shared is None else self.shared(h))
+
+
+class SiluGluMLP(torch.nn.Module):
+    def __init__(self, gate_up_proj: HymetaLinear, down_proj: HymetaLinear):
+        """``gate_up_proj``: rows = gate, then up (with their biases)."""
+        super().__init__()
+        self.gate_up_proj, self.down_proj = gate_up_proj, down_proj
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(hip_ops.silu_mul(self.gate_up_proj(h)))
+
+
+class Relu2RoutedMoE(torch.nn.Module):
+    def __init__(self, router_weight: torch.Tensor, router_bias: Optional[torch.Tensor], w1: torch.Tensor, w2: torch.Tensor, top_k: int):
+        """``w1 [E, I, H]`` (up projections), ``w2 [E, H, I]``."""
+        super().__init__()
+        self.register_buffer("router_weight", router_weight.float().contiguous())     # the router runs in fp32
+        self.register_buffer("router_bias", None if router_bias is None else router_bias.float().contiguous())
+        self.register_buffer("w1", w1.contiguous())
+        self.register_buffer("w2", w2.contiguous())
+        self.top_k = int(top_k)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return hip_ops.moe_routed_forward(h, self.router_weight, self.router_bias, self.w1, self.w2, self.top_k,
+                                          hip_ops.ROUTE_SOFTMAX_CHOSEN, 1.0, "relu2")

@@ -26,6 +26,11 @@ def _geponex_config(model_dir: str):
     return GeponexConfig.from_pretrained(model_dir)
 
 
+def _lidizen_config(model_dir: str):
+    from .models.configuration_lidizen import LidizenConfig
+    return LidizenConfig.from_pretrained(model_dir)
+
+
 def _gla_swa_config(model_dir: str):
     from .model_for_7B.configuration_gla_swa import GLAswaConfig
     with open(os.path.join(model_dir, "config.json")) as f:
@@ -38,6 +43,8 @@ register("Sonuzen", "vllm_hymeta.models.modeling_sonuzen:SonuzenForCausalLM", _s
 register("SonuzenForCausalLM", "vllm_hymeta.models.modeling_sonuzen:SonuzenForCausalLM", _sonuzen_config)
 register("Geponex", "vllm_hymeta.models.modeling_geponex:GeponexForCausalLM", _geponex_config)
 register("GeponexForCausalLM", "vllm_hymeta.models.modeling_geponex:GeponexForCausalLM", _geponex_config)
+register("Lidizen", "vllm_hymeta.models.modeling_lidizen:LidizenForCausalLM", _lidizen_config)
+register("LidizenForCausalLM", "vllm_hymeta.models.modeling_lidizen:LidizenForCausalLM", _lidizen_config)
 register("GLAswaForCausalLM", "vllm_hymeta.model_for_7B.modeling_gla_swa:GLAswaForCausalLM", _gla_swa_config)
 
 
@@ -69,6 +76,8 @@ _KERNEL_SOURCES = {
                            "tall_gemm"),
     "GeponexForCausalLM": ("api_misc", "norm_conv", "post_norm", "latent_attn", "sink_attn", "lightning", "gated_ops", "moe_sigmoid",
                            "moe_table", "moe", "glue", "dense_gemm", "stream_gemm", "tall_gemm"),
+    "LidizenForCausalLM": ("api_misc", "hyper_stream", "talk_attn", "sink_attn", "gated_ops", "moe_sigmoid", "moe_table", "moe", "glue",
+                           "dense_gemm", "stream_gemm", "tall_gemm"),
 }
 
 
