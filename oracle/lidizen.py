@@ -233,3 +233,27 @@ def lidizen_random_weights(cfg: dict, seed: int = 0, std: float = 1.0) -> Dict[s
                 w[f"{p}hc{q}.out"] = rnd(S, scale=0.3, mean=0.7)
                 w[f"{p}hc{q}.mix"] = (torch.eye(S) + torch.randn(S, S, generator=g) * 0.15 * std).to(torch.bfloat16).float()
     return w
+
+
+# ------------------------------------------------------------------------------------------------ kernel-level statements
+def shared_key_attention_ref(q: torch.Tensor, rows: torch.Tensor, num_kv_heads: int, v_dim: int, scale: float, first_pos: int,
+                             size: Optional[int], keep_first: int) -> torch.Tensor:
+    """``q [n, H, Dk]`` are the queries at positions ``first_pos ..``; ``rows [L, Dk + G Dv]`` hold one key for all heads
+    followed by the G values.  Query head h reads value ``h // (H / G)``.  Returns ``[n, H, Dv]``."""
+    n, H, Dk = q.shape
+    L = rows.shape[0]
+    keys, vals = rows[:, :Dk], rows[:, Dk:].reshape(L, num_kv_heads, v_dim)
+    out = torch.zeros(n, H, v_dim, dtype=q.dtype)
+    for r in range(n):
+        i = first_pos + r
+        js = [j for j in range(i + 1) if size is None or i - j < size or j < keep_first]
+        for h in range(H):
+            p = torch.softmax((keys[js] @ q[r, h]) * scale, 0)
+            out[r, h] = p @ vals[js, h // (H // num_kv_heads)]
+    return out
+
+
+def hyper_step_ref(xs: torch.Tensor, y: Optional[torch.Tensor], mix: torch.Tensor, out_w: torch.Tensor) -> torch.Tensor:
+    """``xs [T, S, W]``: every stream rebuilt from the old ones, ``x_t = sum_s mix[s, t] x_s + out_w[t] y``."""
+    new = torch.einsum("st,nsw->ntw", mix, xs)
+    return new if y is None else new + out_w[None, :, None] * y[:, None, :]

@@ -192,9 +192,11 @@ struct MfmaSmem {
 // the same 8 channels of 4 consecutive keys (4 chunks), which are 8 runs of 4 keys in the transposed image, one 8-byte
 // store each.  The 4-key groups of a channel are permuted by the channel's chunk number (XOR), which spreads the stores
 // of threads that hold the same keys over the banks; the reader applies the same permutation.
-// VinK: a head's part of a cache row is its key alone (D elements), whose first DV elements are also its value.
-template <int D, int DV, int Threads, bool VinK>
+// Layout (enum hymeta_kv_layout).  VALUE_IN_KEY: a head's part of a cache row is its key alone (D elements), whose first DV
+// elements are also its value.  SHARED_KEY: a row is one key of D elements for all heads, then num_kv_heads values of DV.
+template <int D, int DV, int Threads, int Layout>
 struct TileStage {
+  static constexpr bool VinK = Layout == HYMETA_KV_VALUE_IN_KEY, Shared = Layout == HYMETA_KV_SHARED_KEY;
   static constexpr int kKeyChunksPerRow = D / 8, kValChunksPerRow = DV / 8;
   static constexpr int kKeyChunks = kTileKeys * kKeyChunksPerRow;
   static constexpr int kKeyPerThread = (kKeyChunks + Threads - 1) / Threads;
@@ -221,8 +223,8 @@ struct TileStage {
     Pages p;
     p.cache = static_cast<const uint16_t*>(a.kv_cache);
     p.bt = bt;
-    p.row_elems = static_cast<int64_t>(a.num_kv_heads) * kHeadElems;
-    p.head_off = static_cast<int64_t>(g) * kHeadElems;
+    p.row_elems = Shared ? D + static_cast<int64_t>(a.num_kv_heads) * DV : static_cast<int64_t>(a.num_kv_heads) * kHeadElems;
+    p.head_off = Shared ? 0 : static_cast<int64_t>(g) * kHeadElems;
     p.shift = __builtin_ctz(a.block_size);
     p.mask = a.block_size - 1;
     p.whole = a.block_size >= kTileKeys;
@@ -344,7 +346,7 @@ __device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSm
         if (Masked) {
           const int j = j0 + 16 * (ks_lo + ks) + 4 * g4 + r;
           const int first = a.window_left >= 0 ? pos - a.window_left : 0;
-          sc = (j <= pos && j >= first) ? sc : -INFINITY;
+          sc = (j <= pos && (j >= first || j < a.keep_first)) ? sc : -INFINITY;
         }
         s[rb][ks][r] = sc;
         mx = fmaxf(mx, sc);
@@ -423,7 +425,7 @@ template <int RB, int Waves> struct PrefillShape { static constexpr int kRows = 
 
 // Portions of prompts: grid = (tiles of 16 RB rows per wave, heads, sequences); a wave holds RB blocks of 16 rows; sequences with
 // one row are left to the decode form.
-template <int D, int DV, int RB, bool VinK>
+template <int D, int DV, int RB, int Layout>
 __global__ __launch_bounds__(64 * PrefillWaves<D>::value) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a, ValueSlice vs) {
   constexpr int kPrefillWaves = PrefillWaves<D>::value;
   constexpr int kRows = PrefillShape<RB, kPrefillWaves>::kRows;
@@ -456,19 +458,25 @@ __global__ __launch_bounds__(64 * PrefillWaves<D>::value) void sink_attention_pr
   const int wave_last = ctx + min(q, wrow + 16 * RB) - 1;
   int j_first = 0;
   if (a.window_left >= 0) j_first = max(0, ctx + static_cast<int>(blockIdx.x) * kRows - a.window_left) / kTileKeys * kTileKeys;
+  // the tiles of the kept first keys that lie before the window's first tile come first, then the window's
+  const int keep_end = a.window_left >= 0 ? min((a.keep_first + kTileKeys - 1) / kTileKeys * kTileKeys, j_first) : 0;
+  const int j_start = keep_end > 0 ? 0 : j_first;
+  auto next = [&](int j0) { return (j0 < keep_end && j0 + kTileKeys >= keep_end) ? j_first : j0 + kTileKeys; };
   // two LDS images: while the waves multiply tile t out of one, tile t + 1 goes into the other and the loads of tile
   // t + 2 are in flight; one barrier per tile
-  TileStage<D, DV, 64 * kPrefillWaves, VinK> stage;
-  if (VinK) stage.value_at = vs.first;
-  stage.issue(a, bt, g, j_first, block_last);
+  TileStage<D, DV, 64 * kPrefillWaves, Layout> stage;
+  if (Layout == HYMETA_KV_VALUE_IN_KEY) stage.value_at = vs.first;
+  if (Layout == HYMETA_KV_SHARED_KEY) stage.value_at = D + g * DV;
+  stage.issue(a, bt, g, j_start, block_last);
   stage.commit(sm[0]);
-  if (kImages == 2 && j_first + kTileKeys <= block_last) stage.issue(a, bt, g, j_first + kTileKeys, block_last);
+  if (kImages == 2 && next(j_start) <= block_last) stage.issue(a, bt, g, next(j_start), block_last);
   __syncthreads();
   if constexpr (kImages == 2) {
     int buf = 0;
-    for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys, buf ^= 1) {
-      if (j0 + kTileKeys <= block_last) stage.commit(sm[buf ^ 1]);
-      if (j0 + 2 * kTileKeys <= block_last) stage.issue(a, bt, g, j0 + 2 * kTileKeys, block_last);
+    for (int j0 = j_start; j0 <= block_last; j0 = next(j0), buf ^= 1) {
+      const int j1 = next(j0), j2 = next(j1);
+      if (j1 <= block_last) stage.commit(sm[buf ^ 1]);
+      if (j2 <= block_last) stage.issue(a, bt, g, j2, block_last);
       if (wrow < q && j0 <= wave_last) {
         // tiles wholly before the wave's first row (and no window) need no mask: every key is visible to every row
         if (a.window_left < 0 && j0 + kTileKeys - 1 <= ctx + wrow) attend_tile<D, DV, RB, 4, false>(w, sm[buf], a, j0, 0);
@@ -479,9 +487,9 @@ __global__ __launch_bounds__(64 * PrefillWaves<D>::value) void sink_attention_pr
   } else {
     // one image (tiles of long rows): the next tile's loads are in flight while this one is multiplied and go into LDS
     // behind a barrier
-    for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys) {
-      const bool more = j0 + kTileKeys <= block_last;
-      if (more) stage.issue(a, bt, g, j0 + kTileKeys, block_last);
+    for (int j0 = j_start; j0 <= block_last; j0 = next(j0)) {
+      const bool more = next(j0) <= block_last;
+      if (more) stage.issue(a, bt, g, next(j0), block_last);
       if (wrow < q && j0 <= wave_last) {
         if (a.window_left < 0 && j0 + kTileKeys - 1 <= ctx + wrow) attend_tile<D, DV, RB, 4, false>(w, sm[0], a, j0, 0);
         else attend_tile<D, DV, RB, 4, true>(w, sm[0], a, j0, 0);
@@ -532,7 +540,7 @@ struct DecodeMerge {
 // Decode: a workgroup per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads; the
 // four waves share the staged tiles and take a 16-key subtile each.  Every wave writes its (maximum, denominator,
 // weighted values) per head; the combine kernel merges them and the sink.
-template <int D, int DV, int RB, bool VinK>
+template <int D, int DV, int RB, int Layout>
 __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split, ValueSlice vs) {
   constexpr int kImages = DecodeImages<D, DV>::value;
   __shared__ MfmaSmem<D, DV> sm[kImages];
@@ -543,10 +551,18 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   const int group = a.num_heads / a.num_kv_heads;
   const int HG = vs.h_count ? vs.h_count : group;            // this launch's rows
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g4 = lane >> 4;
-  int j_lo = split * tiles_per_split * kTileKeys;
-  const int j_hi = min(pos, j_lo + tiles_per_split * kTileKeys - 1);
-  int first = 0;
-  if (a.window_left >= 0) first = max(0, pos - a.window_left);
+  // The sequence's tiles, numbered v = 0 ..: without a window tile v holds the keys from 64 v on, split as the host says.
+  // With a window: the tiles of the kept first keys that lie before the window's first tile, then the window's tiles
+  // (tiles wholly before the window are not read), dealt evenly over the splits.
+  int kept_tiles = 0, window_from = 0, num_tiles = pos / kTileKeys + 1, per = tiles_per_split;
+  if (a.window_left >= 0) {
+    window_from = max(0, pos - a.window_left) / kTileKeys * kTileKeys;
+    kept_tiles = min((a.keep_first + kTileKeys - 1) / kTileKeys * kTileKeys, window_from) / kTileKeys;
+    num_tiles = kept_tiles + (pos - window_from) / kTileKeys + 1;
+    per = (num_tiles + splits - 1) / splits;
+  }
+  const int v_lo = split * per, v_hi = min(num_tiles, v_lo + per) - 1;
+  auto tile = [&](int v) { return v < kept_tiles ? v * kTileKeys : window_from + (v - kept_tiles) * kTileKeys; };
   constexpr bool kMerge = DecodeMerge<D, DV, RB>::value;
   float* part = static_cast<float*>(a.workspace) +
                 (((static_cast<size_t>(s) * a.num_kv_heads + g) * splits + split) * (kMerge ? 1 : kDecodeWaves) + (kMerge ? 0 : wave)) *
@@ -567,21 +583,22 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
   }
-  if (j_lo < first) j_lo = first / kTileKeys * kTileKeys;      // tiles wholly before the window are not read
-  TileStage<D, DV, 64 * kDecodeWaves, VinK> stage;
-  if (VinK) stage.value_at = vs.first;
-  if (j_lo <= j_hi) {
-    stage.issue(a, bt, g, j_lo, j_hi);
+  TileStage<D, DV, 64 * kDecodeWaves, Layout> stage;
+  if (Layout == HYMETA_KV_VALUE_IN_KEY) stage.value_at = vs.first;
+  if (Layout == HYMETA_KV_SHARED_KEY) stage.value_at = D + g * DV;
+  if (v_lo <= v_hi) {
+    stage.issue(a, bt, g, tile(v_lo), pos);
     stage.commit(sm[0]);
-    if (kImages == 2 && j_lo + kTileKeys <= j_hi) stage.issue(a, bt, g, j_lo + kTileKeys, j_hi);
+    if (kImages == 2 && v_lo + 1 <= v_hi) stage.issue(a, bt, g, tile(v_lo + 1), pos);
   }
   __syncthreads();
   if constexpr (kImages == 2) {
     int buf = 0;
-    for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys, buf ^= 1) {
-      if (j0 + kTileKeys <= j_hi) stage.commit(sm[buf ^ 1]);
-      if (j0 + 2 * kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + 2 * kTileKeys, j_hi);
-      if (j0 + 16 * wave <= j_hi) {
+    for (int v = v_lo; v <= v_hi; ++v, buf ^= 1) {
+      const int j0 = tile(v);
+      if (v + 1 <= v_hi) stage.commit(sm[buf ^ 1]);
+      if (v + 2 <= v_hi) stage.issue(a, bt, g, tile(v + 2), pos);
+      if (j0 + 16 * wave <= pos) {
         if (a.window_left < 0 && j0 + kTileKeys - 1 <= pos) attend_tile<D, DV, RB, 1, false>(w, sm[buf], a, j0, wave);
         else attend_tile<D, DV, RB, 1, true>(w, sm[buf], a, j0, wave);
       }
@@ -589,10 +606,11 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
     }
   } else {
     // one image: the next tile's loads are in flight while this one is multiplied and go into LDS behind a barrier
-    for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys) {
-      const bool more = j0 + kTileKeys <= j_hi;
-      if (more) stage.issue(a, bt, g, j0 + kTileKeys, j_hi);
-      if (j0 + 16 * wave <= j_hi) {
+    for (int v = v_lo; v <= v_hi; ++v) {
+      const int j0 = tile(v);
+      const bool more = v + 1 <= v_hi;
+      if (more) stage.issue(a, bt, g, tile(v + 1), pos);
+      if (j0 + 16 * wave <= pos) {
         if (a.window_left < 0 && j0 + kTileKeys - 1 <= pos) attend_tile<D, DV, RB, 1, false>(w, sm[0], a, j0, wave);
         else attend_tile<D, DV, RB, 1, true>(w, sm[0], a, j0, wave);
       }
@@ -694,11 +712,13 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
 // over value slices of 128 (each repeats the scores over the whole key: 1.5 to 2.1 times the matrix work of one pass
 // with accumulators for all the value columns, which do not fit a wave's registers beside the query fragments).
 inline bool mfma_shape(const hymeta_sink_attention_args& a) {
-  if (a.kv_layout == HYMETA_KV_SHARED_KEY || (a.window_left >= 0 && a.keep_first > 0)) return false;
   bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
   if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY)
     dims = ((a.v_dim == 64 || a.v_dim == 128) && (a.head_dim == a.v_dim + 32 || a.head_dim == a.v_dim + 64)) ||
            ((a.v_dim == 256 || a.v_dim == 384 || a.v_dim == 512) && a.head_dim == a.v_dim + 64);      // (in value slices of 128)
+  // one key for all heads: the concatenated keys of 1 / 2 / 4 / 8 key/value heads of 64 or 128
+  if (a.kv_layout == HYMETA_KV_SHARED_KEY)
+    dims = (a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256 || a.head_dim == 512) && (a.v_dim == 64 || a.v_dim == 128);
   return a.act_dtype == HYMETA_BF16 && dims && a.q_stride_t % 8 == 0 &&
          (a.block_size & (a.block_size - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
@@ -716,13 +736,13 @@ inline int decode_splits(int num_seqs, int num_heads, int num_kv_heads, int max_
   return splits > tiles ? (tiles < 1 ? 1 : tiles) : splits;
 }
 
-template <int D, int DV, bool VinK = false>
+template <int D, int DV, int Layout = HYMETA_KV_KEY_THEN_VALUE>
 int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice vs = ValueSlice{0, DV, 0, 0}) {
   if (a.max_query_len > 1) {
     constexpr int kRB = PREFILL_RB;
     constexpr int kRows = PrefillShape<kRB, PrefillWaves<D>::value>::kRows;
     const dim3 grid((a.max_query_len + kRows - 1) / kRows, a.num_heads, a.num_seqs);
-    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB, VinK>), grid, dim3(64 * PrefillWaves<D>::value), 0, st, a, vs);
+    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB, Layout>), grid, dim3(64 * PrefillWaves<D>::value), 0, st, a, vs);
   }
   // sequences with a single row: every step but a pure prompt step has some; a prompt of one token is one too
   const int splits = decode_splits(a.num_seqs, a.num_heads, a.num_kv_heads, a.max_seq_len);
@@ -735,10 +755,10 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice 
     vs.h_count = group - first < kRowsPerWave ? group - first : kRowsPerWave;
     int parts;
     if (vs.h_count <= 16) {
-      hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
+      hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, Layout>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
       parts = splits * (DecodeMerge<D, DV, 1>::value ? 1 : kDecodeWaves);
     } else {
-      hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
+      hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, Layout>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
       parts = splits * (DecodeMerge<D, DV, 2>::value ? 1 : kDecodeWaves);
     }
     hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_kv_heads * vs.h_count), dim3(64), 0, st, a, parts, vs);
@@ -799,17 +819,25 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
     if (!a.workspace || a.workspace_bytes < need) return HYMETA_ERR_WORKSPACE;
     if (a.num_seqs > 65535 || a.num_heads > 65535) return HYMETA_ERR_UNSUPPORTED;
     if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY) {
-      if (a.v_dim == 64) return a.head_dim == 96 ? launch_mfma<96, 64, true>(a, st) : launch_mfma<128, 64, true>(a, st);
-      if (a.v_dim == 128) return a.head_dim == 160 ? launch_mfma<160, 128, true>(a, st) : launch_mfma<192, 128, true>(a, st);
+      if (a.v_dim == 64) return a.head_dim == 96 ? launch_mfma<96, 64, HYMETA_KV_VALUE_IN_KEY>(a, st) : launch_mfma<128, 64, HYMETA_KV_VALUE_IN_KEY>(a, st);
+      if (a.v_dim == 128) return a.head_dim == 160 ? launch_mfma<160, 128, HYMETA_KV_VALUE_IN_KEY>(a, st) : launch_mfma<192, 128, HYMETA_KV_VALUE_IN_KEY>(a, st);
       hymeta_sink_attention_args b = a;
       b.v_dim = 128;
       for (int first = 0; first < a.v_dim; first += 128) {
         const ValueSlice vs{first, a.v_dim, 0, 0};
-        const int rc = a.v_dim == 256 ? launch_mfma<320, 128, true>(b, st, vs) : a.v_dim == 384 ? launch_mfma<448, 128, true>(b, st, vs)
-                                                                                                 : launch_mfma<576, 128, true>(b, st, vs);
+        const int rc = a.v_dim == 256 ? launch_mfma<320, 128, HYMETA_KV_VALUE_IN_KEY>(b, st, vs) : a.v_dim == 384 ? launch_mfma<448, 128, HYMETA_KV_VALUE_IN_KEY>(b, st, vs)
+                                                                                                 : launch_mfma<576, 128, HYMETA_KV_VALUE_IN_KEY>(b, st, vs);
         if (rc != HYMETA_OK) return rc;
       }
       return HYMETA_OK;
+    }
+    if (a.kv_layout == HYMETA_KV_SHARED_KEY) {
+      constexpr int kShared = HYMETA_KV_SHARED_KEY;
+      if (a.v_dim == 64)
+        return a.head_dim == 64 ? launch_mfma<64, 64, kShared>(a, st) : a.head_dim == 128 ? launch_mfma<128, 64, kShared>(a, st)
+             : a.head_dim == 256 ? launch_mfma<256, 64, kShared>(a, st) : launch_mfma<512, 64, kShared>(a, st);
+      return a.head_dim == 64 ? launch_mfma<64, 128, kShared>(a, st) : a.head_dim == 128 ? launch_mfma<128, 128, kShared>(a, st)
+           : a.head_dim == 256 ? launch_mfma<256, 128, kShared>(a, st) : launch_mfma<512, 128, kShared>(a, st);
     }
     if (a.head_dim == 64 && a.v_dim == 64) return launch_mfma<64, 64>(a, st);
     if (a.head_dim == 64 && a.v_dim == 128) return launch_mfma<64, 128>(a, st);
