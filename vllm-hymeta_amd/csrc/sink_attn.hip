@@ -544,7 +544,16 @@ template <int D, int DV, int RB, int Layout>
 __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split, ValueSlice vs) {
   constexpr int kImages = DecodeImages<D, DV>::value;
   __shared__ MfmaSmem<D, DV> sm[kImages];
-  const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
+  int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
+  if (Layout == HYMETA_KV_SHARED_KEY) {
+    // The value groups of a (sequence, split) read the same key tiles.  Workgroups go to the chip's 8 dies (each with an
+    // L2 of its own) round robin by their number: a one-dimensional grid numbered so that those groups follow each other
+    // on ONE die, which then fetches the keys from memory once instead of once per group.
+    const int chunk = blockIdx.x >> 3, die = blockIdx.x & 7;
+    const int pair = (chunk / a.num_kv_heads) * 8 + die;
+    if (pair >= splits * a.num_seqs) return;
+    g = chunk % a.num_kv_heads, s = pair / splits, split = pair % splits;
+  }
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
   const int pos = a.seq_lens[s] - 1;
@@ -748,7 +757,7 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice 
   const int splits = decode_splits(a.num_seqs, a.num_heads, a.num_kv_heads, a.max_seq_len);
   const int tiles = (a.max_seq_len + kTileKeys - 1) / kTileKeys;
   const int tiles_per_split = (tiles + splits - 1) / splits;
-  const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
+  const dim3 grid = Layout == HYMETA_KV_SHARED_KEY ? dim3((splits * a.num_seqs + 7) / 8 * 8 * a.num_kv_heads) : dim3(splits, a.num_kv_heads, a.num_seqs);
   const int group = a.num_heads / a.num_kv_heads;
   for (int first = 0; first < group; first += kRowsPerWave) {
     vs.h_first = first;

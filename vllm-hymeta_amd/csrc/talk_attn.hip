@@ -13,6 +13,8 @@ namespace hymeta {
 namespace {
 
 constexpr int kMaxRotPairs = 512;
+constexpr int kTalkLdsHeads = 64;      // the mix matrix of up to this many heads is read from LDS
+constexpr int kGroupRegs = 16;         // query heads of a group a thread keeps in registers
 
 // grid = tokens; dynamic LDS: (H + G) * D floats (the normed and rotated queries and keys of the token)
 template <typename A>
@@ -21,6 +23,7 @@ __global__ __launch_bounds__(256) void talk_qkv_prep_kernel(hymeta_talk_qkv_prep
   extern __shared__ float s_qk[];
   __shared__ float s_cos[kMaxRotPairs], s_sin[kMaxRotPairs];
   __shared__ float red[4];
+  __shared__ float s_talk[kTalkLdsHeads * kTalkLdsHeads];
   const int t = blockIdx.x, tid = threadIdx.x;
   const int H = a.num_heads, G = a.num_kv_heads, D = a.head_dim, Dv = a.v_dim;
   const int nq = H * D, nk = G * D, nv = G * Dv, group = H / G;
@@ -72,14 +75,38 @@ __global__ __launch_bounds__(256) void talk_qkv_prep_kernel(hymeta_talk_qkv_prep
       A::st(dst + nk + c, r);
     }
   }
+  // a thread takes a column of the shared key (a key/value head's dimension d) and walks the query heads: the group's
+  // queries of that dimension stay in registers, the mix weights are LDS broadcasts, the stores of a wave are consecutive
   elem* qo = static_cast<elem*>(a.q_out) + static_cast<int64_t>(t) * H * nk;
-  for (int idx = tid; idx < H * nk; idx += 256) {
-    const int h = idx / nk, c = idx % nk, kv = c / D, d = c % D;
-    const float* tw = a.talk + static_cast<int64_t>(h) * H + kv * group;
+  const float* talk = a.talk;
+  if (H <= kTalkLdsHeads) {
+    for (int i = tid; i < H * H; i += 256) s_talk[i] = a.talk[i];
+    __syncthreads();
+    talk = s_talk;
+  }
+  for (int c = tid; c < nk; c += 256) {
+    const int kv = c / D, d = c % D;
     const float* q = s_qk + (kv * group) * D + d;
-    float r = 0.f;
-    for (int j = 0; j < group; ++j) r = fmaf(tw[j], q[j * D], r);
-    A::st(qo + idx, r);
+    if (group <= kGroupRegs) {
+      float qv[kGroupRegs];
+#pragma unroll
+      for (int j = 0; j < kGroupRegs; ++j) qv[j] = j < group ? q[j * D] : 0.f;
+      for (int h = 0; h < H; ++h) {
+        const float* tw = talk + h * H + kv * group;
+        float r = 0.f;
+#pragma unroll
+        for (int j = 0; j < kGroupRegs; ++j)
+          if (j < group) r = fmaf(tw[j], qv[j], r);
+        A::st(qo + static_cast<int64_t>(h) * nk + c, r);
+      }
+    } else {
+      for (int h = 0; h < H; ++h) {
+        const float* tw = talk + h * H + kv * group;
+        float r = 0.f;
+        for (int j = 0; j < group; ++j) r = fmaf(tw[j], q[j * D], r);
+        A::st(qo + static_cast<int64_t>(h) * nk + c, r);
+      }
+    }
   }
 }
 
