@@ -1460,7 +1460,7 @@ int hymeta_embed_pair(const hymeta_embed_pair_args* args, hymeta_stream_t stream
  *   (y != NULL)      x_t <- sum_s mix[s, t] x_s + out_w[t] * y        all streams at once from the old ones
  *   (h_out != NULL)  h = norm(sum_s in_w[s] x_s)                     from the new streams, act_dtype
  * norm: layer norm times norm_weight (norm_weight NULL: the weighted sum itself).  One stream with mix = out_w = in_w =
- * 1 is the plain residual add followed by the next sublayer's norm.  streams <= 8, width <= 8192. */
+ * 1 is the plain residual add followed by the next sublayer's norm.  streams <= HYMETA_MAX_STREAMS, width <= 8192. */
 typedef struct hymeta_hyper_stream_args {
   uint32_t struct_size;
   float* x;                    /* [num_tokens, streams, width] */
@@ -1474,7 +1474,7 @@ typedef struct hymeta_hyper_stream_args {
   float eps;
   int64_t y_stride_t;
 } hymeta_hyper_stream_args;
-#define HYMETA_MAX_STREAMS 8
+#define HYMETA_MAX_STREAMS 16
 int hymeta_hyper_stream(const hymeta_hyper_stream_args* args, hymeta_stream_t stream);
 
 /* Between the fused q | k | v projection and hymeta_sink_attention with HYMETA_KV_SHARED_KEY, per token, one launch:

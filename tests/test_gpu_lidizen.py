@@ -107,7 +107,7 @@ def test_pair_embedding_in_portions_carries_the_previous_token(dtype, width, cop
 
 # --------------------------------------------------------------------------- residual streams
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("S,width", [(1, 48), (2, 256), (3, 600), (4, 1024), (8, 130), (5, 2048)])
+@pytest.mark.parametrize("S,width", [(1, 48), (2, 256), (3, 600), (4, 1024), (8, 130), (5, 2048), (11, 96), (4, 3584)])
 def test_streams_write_and_read_in_one_launch(dtype, S, width):
     from vllm_hymeta import hip_ops
     g = torch.Generator().manual_seed(S * 1000 + width)
@@ -188,6 +188,26 @@ def test_attention_over_a_shared_key_with_a_window_that_keeps_the_first_keys(dty
     got = _attend(qs, cache, perm, G, Dk, Dv, scale, [1, 1, 1, 1, 80], pos[:4] + [150], window, keep, page)
     want = torch.cat([ref[p:p + 1] for p in pos[:4]] + [ref[150:230]])
     assert rel_err(got, want) < tol
+
+
+@pytest.mark.parametrize("dtype,H,G,Dk,Dv", [(torch.float32, 4, 2, 48, 24), (torch.bfloat16, 8, 2, 128, 64), (torch.bfloat16, 6, 1, 64, 128), (torch.bfloat16, 4, 4, 96, 40)])
+def test_a_window_far_into_a_long_sequence(dtype, H, G, Dk, Dv):
+    """2100 keys on scattered pages, a window of 96 and 4 kept keys: the whole prompt, a late portion, and single rows at
+    tile borders far from the start (most of a decode launch's key splits see no key at all)."""
+    g = torch.Generator().manual_seed(Dk)
+    L, window, keep, page = 2100, 96, 4, 64
+    rows = torch.randn(L, Dk + G * Dv, generator=g).to(dtype)
+    q = torch.randn(L, H, Dk, generator=g).to(dtype)
+    scale = Dk ** -0.5 * 2.0
+    ref = shared_key_attention_ref(q.double(), rows.double(), G, Dv, scale, 0, window, keep)
+    cache, perm = _paged(rows, dtype, page, seed=L)
+    tol = 3e-6 if dtype == torch.float32 else 6e-3
+    qd = q.to(DEV)
+    assert rel_err(_attend(qd, cache, perm, G, Dk, Dv, scale, [L], [0], window, keep, page), ref) < tol
+    assert rel_err(_attend(qd[1900:2077], cache, perm, G, Dk, Dv, scale, [177], [1900], window, keep, page), ref[1900:2077]) < tol
+    pos = [2099, 2048, 2047, 1983, 1152, 99, 96, 95]
+    got = _attend(torch.cat([qd[p:p + 1] for p in pos]), cache, perm, G, Dk, Dv, scale, [1] * len(pos), pos, window, keep, page)
+    assert rel_err(got, torch.cat([ref[p:p + 1] for p in pos])) < tol
 
 
 @pytest.mark.parametrize("dtype,Dk,Dv", [(torch.float32, 48, 24), (torch.bfloat16, 128, 64), (torch.bfloat16, 256, 128), (torch.bfloat16, 40, 16)])
@@ -558,3 +578,81 @@ def test_trace_runner_and_generate_command_lines(tmp_path):
             assert t == int(logits.argmax())
         toks.append(t)
     assert len(line["output"]) == 3
+
+
+def _random_model(seed):
+    """Sizes drawn at random: head counts, group sizes, key and value sizes (also such that a layer's concatenated keys
+    and its values take the matrix-core kernels), windows around a page and a tile, kept keys, streams, feed-forwards."""
+    import random
+    r = random.Random(seed)
+    width = r.choice([24, 40, 64, 96, 128, 200])
+    layers = []
+    blend_shape = None
+    for _ in range(r.randint(1, 4)):
+        G = r.choice([1, 2, 3, 4])
+        H = G * r.choice([1, 2, 3, 5])
+        if r.random() < 0.4:
+            D, Dv = r.choice([(64 // G if G in (1, 2, 4) else 32, 64), (128 // G if G in (1, 2, 4) else 64, 64), (64, 128), (32, 64)])
+        else:
+            D, Dv = 2 * r.randint(2, 20), r.randint(3, 40)
+        v_mix = r.random() < 0.6
+        if v_mix:
+            if blend_shape is None:
+                blend_shape = (G, Dv)
+            elif blend_shape != (G, Dv):
+                H, (G, Dv) = blend_shape[0] * r.choice([1, 2, 4]), blend_shape
+        size = r.choice([1, 2, 7, 15, 16, 17, 63, 64, 65, 100, 128, 1000])
+        mixer = attention_config(heads=H, kv_heads=G, dim=D, vdim=Dv, size=size, keep_first=r.choice([0, 0, 1, 3, 16, 64, 70]),
+                                 rot_dims=r.choice([0, 2, D // 2 * 2, D // 4 * 2]), base=r.choice([10.0, 10000.0, 500000.0]),
+                                 scale=r.choice([D ** -0.5, 0.3, 0.05]), v_mix=v_mix)
+        kind = r.choice(["dense", "moe", "moe", None])
+        mlp = None if kind is None else {"kind": "dense", "ff": r.choice([16, 72, 128])} if kind == "dense" else _moe(r.randint(1, 9), 1, r.choice([8, 40, 64, 128]))
+        if mlp and mlp["kind"] == "moe":
+            mlp["router"]["top"] = r.randint(1, mlp["router"]["experts"])
+        layers.append(_layer(mixer, mlp))
+    bigram = None if r.random() < 0.2 else (r.choice([1, 7, 251, 4099]), r.randint(0, 40), r.randint(1, 40))
+    return lidizen_config(vocab=r.choice([50, 130]), width=width, layers=layers, streams=r.choice([0, 1, 2, 3, 4, 6]), eps=r.choice([1e-5, 1e-6, 1e-3]),
+                          bigram=bigram)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_models_of_random_sizes_under_the_engine(seed):
+    """fp32: a prompt of 210 tokens in one step, then in portions and single tokens beside a second request, against the
+    oracle; bf16 (every expert chosen): the same schedule against the one-step result."""
+    cfg = _random_model(seed)
+    weights = lidizen_random_weights(cfg, seed=seed)
+    V = cfg["vocab"]
+    a, b = _tokens(210, V, 100 + seed), _tokens(75, V, 200 + seed)
+    ra, rb = lidizen_ref(cfg, weights, a), lidizen_ref(cfg, weights, b)
+    page = 64 if seed % 2 else 16
+    plan = [[(0, 3)], [(0, 64), (1, 2)], [(0, 1), (1, 1)], [(0, 62), (1, 70)], [(0, 1), (1, 1)], [(0, 2), (1, 1)], [(0, 77)]]
+    for dtype in (torch.float32, torch.bfloat16):
+        c = cfg
+        if dtype == torch.bfloat16:
+            import copy
+            c = copy.deepcopy(cfg)
+            for entry in c["layers"]:
+                if entry["mlp"] and entry["mlp"]["kind"] == "moe":
+                    entry["mlp"]["router"]["top"] = entry["mlp"]["router"]["experts"]
+        exact = dtype == torch.float32
+        eng = build_engine(c, weights, dtype, max_tokens=448, block_size=page, max_num_seqs=2)
+        wa = eng.run_batch([("wa", a, list(range(len(a))))])
+        eng.finish_request("wa")
+        if exact:
+            assert rel_err(wa, ra) < 5e-5
+        seqs, at, got = {0: a, 1: b}, {0: 0, 1: 0}, {0: [], 1: []}
+        for step in plan:
+            out = eng.run_batch([(f"r{k}", seqs[k][at[k]:at[k] + n], list(range(n))) for k, n in step])
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n])
+                row += n
+                at[k] += n
+                if at[k] == len(seqs[k]):
+                    eng.finish_request(f"r{k}")
+        assert at == {0: 210, 1: 75} and not eng.requests
+        ga, gb = torch.cat(got[0]), torch.cat(got[1])
+        if exact:
+            assert rel_err(ga, ra) < 5e-5 and rel_err(gb, rb) < 5e-5
+        else:
+            assert rows_close(ga, wa, 0.1, False)

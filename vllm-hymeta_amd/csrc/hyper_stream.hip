@@ -239,7 +239,7 @@ __global__ __launch_bounds__(256) void hyper_stream_kernel(hymeta_hyper_stream_a
   }
 }
 
-// Any width (and pointers that are not 16-byte aligned): a column per thread and round, the weighted sum through LDS
+// Any width, more than 8 streams, pointers that are not 16-byte aligned: a column per thread and round, the weighted sum through LDS
 // (dynamic: width floats) between the rounds.
 template <typename A>
 __global__ __launch_bounds__(256) void hyper_stream_any_kernel(hymeta_hyper_stream_args a) {
@@ -308,7 +308,7 @@ void launch_hyper_stream(const hymeta_hyper_stream_args& a, hipStream_t st) {
   auto fours = [&](const void* p, int64_t stride, int b) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % (4 * b) == 0 && stride % 4 == 0); };
   const bool vec = a.width % 4 == 0 && fours(a.x, a.width, 4) && fours(a.y, a.y_stride_t, bytes) && fours(a.h_out, a.width, bytes) &&
                    fours(a.norm_weight, 4, 4);
-  if (!vec) {
+  if (!vec || a.streams > 8) {
     hipLaunchKernelGGL(hyper_stream_any_kernel<A>, dim3(a.num_tokens), dim3(256), a.h_out ? a.width * sizeof(float) : 0, st, a);
     return;
   }

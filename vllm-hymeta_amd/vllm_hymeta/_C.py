@@ -32,7 +32,7 @@ KV_SHARED_KEY = 2
 GLU_NONE, GLU_SILU, GLU_CLAMPED, GLU_RELU2 = 0, 1, 2, 3
 ACT_CLAMPED_GLU, ACT_XIELU, ACT_SIGMOID_MUL, ACT_SILU_MUL, ACT_RELU2 = 0, 1, 2, 3, 4
 ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN = 0, 1
-MAX_STREAMS = 8
+MAX_STREAMS = 16
 LIGHTNING_CHUNK = 64
 CONV_MAX_TAPS = 8
 
