@@ -25,7 +25,7 @@ def lidizen_config(width, heads, kv_heads, dim, layers, experts, top, ff, vocab,
         mlp = dict(kind="dense", ff=top * ff) if kind == "dense" else dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top))
         ls.append(dict(type="attention", mixer=mixer, mlp=mlp))
     return dict(architecture="Lidizen", vocab=vocab, width=width, streams=streams, layers=ls, norm=dict(eps=1e-5),
-                embedding=dict(bigram=dict(buckets=65521, mul_prev=31, mul_cur=17)))
+                embedding=dict(bigram=dict(buckets=65521, mul_prev=37, mul_cur=19)))
 
 
 def lidizen_checkpoint(cfg, dev, seed=0):
@@ -166,7 +166,7 @@ def kernel_table(dev, W, H, G, D, B, ctx, L, E, top, ff, window, keep, S=4):
         table, pair = rnd(32768, W), rnd(65522, W)
         prev = torch.zeros(max(B, 4), dtype=torch.int32, device=dev)
         lay = (qsl, ones, sidx) if T == B else (i32([0, T]), i32([0]), i32([1]))
-        add(f"embed_pair ({S} streams) T={T}", lambda: hip_ops.embed_pair(ids, table, pair, wn, 1e-5, S, 65521, 31, 17, prev, *lay), nbytes=T * W * (4 + S * 4))
+        add(f"embed_pair ({S} streams) T={T}", lambda: hip_ops.embed_pair(ids, table, pair, wn, 1e-5, S, 65521, 37, 19, prev, *lay), nbytes=T * W * (4 + S * 4))
         add(f"embed_rows (Sonuzen) T={T}", lambda: hip_ops.embed_rows(ids, table), nbytes=T * W * (2 + 4))
         gu = rnd(T, 2 * top * ff)
         add(f"silu_mul T={T}", lambda: hip_ops.silu_mul(gu), nbytes=T * top * ff * 6)

@@ -1501,6 +1501,7 @@ typedef struct hymeta_talk_qkv_prep_args {
   int32_t num_tokens, num_seqs, num_heads, num_kv_heads, head_dim, v_dim, rot_dims, block_size, act_dtype;
   float eps, v_blend;
   int64_t num_blocks, qkv_stride_t, v_other_stride_t;
+  const int64_t* positions;    /* [num_tokens] or NULL: a row's position is its sequence's length minus the rows behind it */
 } hymeta_talk_qkv_prep_args;
 int hymeta_talk_qkv_prep(const hymeta_talk_qkv_prep_args* args, hymeta_stream_t stream);
 

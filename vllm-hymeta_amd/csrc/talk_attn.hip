@@ -16,19 +16,34 @@ constexpr int kMaxRotPairs = 512;
 constexpr int kTalkLdsHeads = 64;      // the mix matrix of up to this many heads is read from LDS
 constexpr int kGroupRegs = 16;         // query heads of a group a thread keeps in registers
 
-// grid = tokens; dynamic LDS: (H + G) * D floats (the normed and rotated queries and keys of the token)
-template <typename A>
+__device__ __forceinline__ void store_pair(uint16_t* p, float a, float b) { *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(a, b); }
+__device__ __forceinline__ void store_pair(float* p, float a, float b) { *reinterpret_cast<u32x2*>(p) = u32x2{__float_as_uint(a), __float_as_uint(b)}; }
+
+// grid = tokens; dynamic LDS: (H + G) * D floats (the normed and rotated queries and keys of the token).
+// Vec: the row in fours of columns (aligned, H D and G D in whole fours) and the mixed queries in pairs (D even).
+template <typename A, bool Vec>
 __global__ __launch_bounds__(256) void talk_qkv_prep_kernel(hymeta_talk_qkv_prep_args a) {
   typedef typename A::elem elem;
-  extern __shared__ float s_qk[];
+  extern __shared__ __attribute__((aligned(16))) float s_qk[];
   __shared__ float s_cos[kMaxRotPairs], s_sin[kMaxRotPairs];
   __shared__ float red[4];
   __shared__ float s_talk[kTalkLdsHeads * kTalkLdsHeads];
   const int t = blockIdx.x, tid = threadIdx.x;
   const int H = a.num_heads, G = a.num_kv_heads, D = a.head_dim, Dv = a.v_dim;
   const int nq = H * D, nk = G * D, nv = G * Dv, group = H / G;
-  const int s = seq_of_row(a.query_start_loc, a.num_seqs, t);
-  const int pos = max(a.seq_lens[s] - (a.query_start_loc[s + 1] - t), 0);
+  // what does not depend on the token goes first: the mix matrix is in LDS long before the mix reads it
+  const float* talk = a.talk;
+  if (H <= kTalkLdsHeads) {
+    for (int i = tid; i < H * H; i += 256) s_talk[i] = a.talk[i];
+    talk = s_talk;
+  }
+  int pos;
+  if (a.positions) {
+    pos = static_cast<int>(a.positions[t]);
+  } else {
+    const int s = seq_of_row(a.query_start_loc, a.num_seqs, t);
+    pos = max(a.seq_lens[s] - (a.query_start_loc[s + 1] - t), 0);
+  }
   const elem* row = static_cast<const elem*>(a.qkv) + static_cast<int64_t>(t) * a.qkv_stride_t;
   // angles in double precision, brought into [-pi, pi]; the functions are the fp32 ones on the remainder
   for (int i = tid; i < a.rot_dims / 2; i += 256) {
@@ -39,10 +54,20 @@ __global__ __launch_bounds__(256) void talk_qkv_prep_kernel(hymeta_talk_qkv_prep
     s_sin[i] = sinf(r);
   }
   float ssq = 0.f, ssk = 0.f;
-  for (int c = tid; c < nq + nk; c += 256) {
-    const float v = A::ld(row + c);
-    s_qk[c] = v;
-    if (c < nq) ssq = fmaf(v, v, ssq); else ssk = fmaf(v, v, ssk);
+  if (Vec) {
+    for (int c = 4 * tid; c < nq + nk; c += 1024) {
+      float v[4];
+      A::ld4(row + c, v);
+      *reinterpret_cast<f32x4*>(&s_qk[c]) = f32x4{v[0], v[1], v[2], v[3]};
+      const float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+      if (c < nq) ssq += ss; else ssk += ss;
+    }
+  } else {
+    for (int c = tid; c < nq + nk; c += 256) {
+      const float v = A::ld(row + c);
+      s_qk[c] = v;
+      if (c < nq) ssq = fmaf(v, v, ssq); else ssk = fmaf(v, v, ssk);
+    }
   }
   const float inv_q = 1.f / sqrtf(block_sum<4>(ssq, red) / static_cast<float>(nq) + a.eps);
   const float inv_k = 1.f / sqrtf(block_sum<4>(ssk, red) / static_cast<float>(nk) + a.eps);
@@ -75,38 +100,58 @@ __global__ __launch_bounds__(256) void talk_qkv_prep_kernel(hymeta_talk_qkv_prep
       A::st(dst + nk + c, r);
     }
   }
-  // a thread takes a column of the shared key (a key/value head's dimension d) and walks the query heads: the group's
-  // queries of that dimension stay in registers, the mix weights are LDS broadcasts, the stores of a wave are consecutive
+  // a thread takes columns of the shared key (a key/value head's dimension d; two neighbours in the Vec form) and walks
+  // the query heads: the group's queries of those columns stay in registers, the mix weights are LDS broadcasts, the
+  // stores of a wave are consecutive
   elem* qo = static_cast<elem*>(a.q_out) + static_cast<int64_t>(t) * H * nk;
-  const float* talk = a.talk;
-  if (H <= kTalkLdsHeads) {
-    for (int i = tid; i < H * H; i += 256) s_talk[i] = a.talk[i];
-    __syncthreads();
-    talk = s_talk;
-  }
-  for (int c = tid; c < nk; c += 256) {
+  constexpr int kCols = Vec ? 2 : 1;
+  for (int c = kCols * tid; c < nk; c += kCols * 256) {
     const int kv = c / D, d = c % D;
     const float* q = s_qk + (kv * group) * D + d;
     if (group <= kGroupRegs) {
-      float qv[kGroupRegs];
+      float qv[kGroupRegs][kCols];
 #pragma unroll
-      for (int j = 0; j < kGroupRegs; ++j) qv[j] = j < group ? q[j * D] : 0.f;
+      for (int j = 0; j < kGroupRegs; ++j)
+#pragma unroll
+        for (int e = 0; e < kCols; ++e) qv[j][e] = j < group ? q[j * D + e] : 0.f;
       for (int h = 0; h < H; ++h) {
         const float* tw = talk + h * H + kv * group;
-        float r = 0.f;
+        float r[kCols] = {};
 #pragma unroll
         for (int j = 0; j < kGroupRegs; ++j)
-          if (j < group) r = fmaf(tw[j], qv[j], r);
-        A::st(qo + static_cast<int64_t>(h) * nk + c, r);
+          if (j < group) {
+            const float wj = tw[j];
+#pragma unroll
+            for (int e = 0; e < kCols; ++e) r[e] = fmaf(wj, qv[j][e], r[e]);
+          }
+        if (Vec) store_pair(qo + static_cast<int64_t>(h) * nk + c, r[0], r[kCols - 1]);
+        else A::st(qo + static_cast<int64_t>(h) * nk + c, r[0]);
       }
     } else {
       for (int h = 0; h < H; ++h) {
         const float* tw = talk + h * H + kv * group;
-        float r = 0.f;
-        for (int j = 0; j < group; ++j) r = fmaf(tw[j], q[j * D], r);
-        A::st(qo + static_cast<int64_t>(h) * nk + c, r);
+        float r[kCols] = {};
+        for (int j = 0; j < group; ++j)
+#pragma unroll
+          for (int e = 0; e < kCols; ++e) r[e] = fmaf(tw[j], q[j * D + e], r[e]);
+        if (Vec) store_pair(qo + static_cast<int64_t>(h) * nk + c, r[0], r[kCols - 1]);
+        else A::st(qo + static_cast<int64_t>(h) * nk + c, r[0]);
       }
     }
+  }
+}
+
+template <typename A>
+void launch_talk_qkv_prep(const hymeta_talk_qkv_prep_args& a, size_t lds, hipStream_t st) {
+  const int bytes = A::kDtype == HYMETA_BF16 ? 2 : 4;
+  const bool vec = a.head_dim % 4 == 0 && reinterpret_cast<uintptr_t>(a.qkv) % (4 * bytes) == 0 && a.qkv_stride_t % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(a.q_out) % (2 * bytes) == 0;
+  if (vec) {
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(talk_qkv_prep_kernel<A, true>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    hipLaunchKernelGGL((talk_qkv_prep_kernel<A, true>), dim3(a.num_tokens), dim3(256), lds, st, a);
+  } else {
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(talk_qkv_prep_kernel<A, false>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    hipLaunchKernelGGL((talk_qkv_prep_kernel<A, false>), dim3(a.num_tokens), dim3(256), lds, st, a);
   }
 }
 
@@ -127,19 +172,14 @@ extern "C" int hymeta_talk_qkv_prep(const hymeta_talk_qkv_prep_args* args, hymet
   const int64_t floats = static_cast<int64_t>(a.num_heads + a.num_kv_heads) * a.head_dim;
   if (a.rot_dims / 2 > kMaxRotPairs || floats * 4 > 96 * 1024) return HYMETA_ERR_UNSUPPORTED;
   if (a.num_tokens == 0 || a.num_seqs == 0) return HYMETA_OK;
-  if (!a.qkv || !a.q_weight || !a.k_weight || !a.talk || !a.q_out || !a.query_start_loc || !a.seq_lens || (a.rot_dims > 0 && !a.rot_freqs))
+  if (!a.qkv || !a.q_weight || !a.k_weight || !a.talk || !a.q_out || (!a.positions && (!a.query_start_loc || !a.seq_lens)) || (a.rot_dims > 0 && !a.rot_freqs))
     return HYMETA_ERR_INVALID_ARG;
   if (a.slot_mapping && !a.kv_cache) return HYMETA_ERR_INVALID_ARG;
   if (a.qkv_stride_t < floats + static_cast<int64_t>(a.num_kv_heads) * a.v_dim) return HYMETA_ERR_INVALID_ARG;
   if (a.v_other && a.v_other_stride_t < static_cast<int64_t>(a.num_kv_heads) * a.v_dim) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
   const size_t lds = static_cast<size_t>(floats) * sizeof(float);
-  if (a.act_dtype == HYMETA_BF16) {
-    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(talk_qkv_prep_kernel<ActBf16>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    hipLaunchKernelGGL(talk_qkv_prep_kernel<ActBf16>, dim3(a.num_tokens), dim3(256), lds, st, a);
-  } else {
-    if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(talk_qkv_prep_kernel<ActF32>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-    hipLaunchKernelGGL(talk_qkv_prep_kernel<ActF32>, dim3(a.num_tokens), dim3(256), lds, st, a);
-  }
+  if (a.act_dtype == HYMETA_BF16) launch_talk_qkv_prep<ActBf16>(a, lds, st);
+  else launch_talk_qkv_prep<ActF32>(a, lds, st);
   return launch_status();
 }

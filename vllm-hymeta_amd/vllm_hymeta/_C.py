@@ -509,6 +509,7 @@ class TalkQkvPrepArgs(_Args):
         ("rot_dims", _i32), ("block_size", _i32), ("act_dtype", _i32),
         ("eps", _f32), ("v_blend", _f32),
         ("num_blocks", _i64), ("qkv_stride_t", _i64), ("v_other_stride_t", _i64),
+        ("positions", _ptr),
     ]
 
 

@@ -2103,13 +2103,14 @@ def hyper_stream_(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torc
 def talk_qkv_prep(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int, q_weight: torch.Tensor,
                   k_weight: torch.Tensor, talk: torch.Tensor, eps: float, rot_dims: int, rot_freqs: Optional[torch.Tensor],
                   kv_cache: torch.Tensor, slot_mapping: torch.Tensor, query_start_loc: torch.Tensor, seq_lens: torch.Tensor,
-                  v_other: Optional[torch.Tensor] = None, v_blend: float = 0.0) -> torch.Tensor:
+                  v_other: Optional[torch.Tensor] = None, v_blend: float = 0.0, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
     """From ``qkv [T, H D + G D + G Dv]``: RMS norms over the whole query and key projections, rotation of the first
     ``rot_dims`` dimensions of every head in interleaved pairs, values blended with ``v_other`` (``(1 - v_blend) v + v_blend
     v_other``), the paged write of ``(keys of all G heads, values of all G heads)`` into ``kv_cache [blocks, block_size, 1,
     G D + G Dv]``; returns the queries mixed across heads, ``[T, H, G D]``: ``out[h, g D + d] = sum_j talk[h, j] q[j, d]``
-    over the query heads ``j`` of group ``g``."""
-    _dev(qkv, q_weight, k_weight, talk, rot_freqs, kv_cache, slot_mapping, query_start_loc, seq_lens, v_other)
+    over the query heads ``j`` of group ``g``.  ``positions`` int64 ``[T]``: the rows' positions where the caller has them
+    (otherwise they follow from ``query_start_loc`` and ``seq_lens``)."""
+    _dev(qkv, q_weight, k_weight, talk, rot_freqs, kv_cache, slot_mapping, query_start_loc, seq_lens, v_other, positions)
     T = qkv.shape[0]
     H, G, D, Dv = num_heads, num_kv_heads, head_dim, v_dim
     _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (H + G) * D + G * Dv and qkv.dtype in _DT,
@@ -2135,5 +2136,8 @@ def talk_qkv_prep(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         _require(v_other.dim() == 2 and v_other.shape == (T, G * Dv) and v_other.stride(1) == 1 and v_other.dtype == qkv.dtype,
                  "v_other must be row-contiguous [T, G Dv] of qkv's type")
         a.v_other, a.v_other_stride_t, a.v_blend = _p(v_other), v_other.stride(0), v_blend
+    if positions is not None:
+        _require(positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T, "positions must be contiguous int64 [T]")
+        a.positions = _p(positions)
     _C.check(_C.load().hymeta_talk_qkv_prep(C.byref(a), _stream(qkv)), "hymeta_talk_qkv_prep")
     return q_out

@@ -67,17 +67,18 @@ class LidizenModel(torch.nn.Module):
         self.blocks = torch.nn.ModuleList()
         self.final_read: Optional[StreamNormRead] = None
 
-    def layout_of(self, attn_metadata, slot_idx: torch.Tensor, token_ids: torch.Tensor) -> StepLayout:
+    def layout_of(self, attn_metadata, slot_idx: torch.Tensor, token_ids: torch.Tensor, positions: Optional[torch.Tensor] = None) -> StepLayout:
         md = attn_metadata
         max_seq = max(md.seq_lens) if md.seq_lens else max(md.max_prefill_seq_len, md.max_decode_seq_len)
         return StepLayout(query_start_loc=md.query_start_loc, context_lens=md.context_lens_tensor, seq_lens=md.seq_lens_tensor,
                           slot_idx=slot_idx, block_tables=md.block_tables, slot_mapping=md.slot_mapping,
-                          max_query_len=int(md.max_query_len or 1), max_seq_len=int(max_seq), token_ids=token_ids)
+                          max_query_len=int(md.max_query_len or 1), max_seq_len=int(max_seq), token_ids=token_ids, positions=positions)
 
     def forward(self, input_ids: torch.Tensor, positions: Optional[torch.Tensor] = None, attn_metadata=None,
                 kv_caches: Optional[List[torch.Tensor]] = None, residual_out: Optional[List[torch.Tensor]] = None,
                 **kwargs) -> torch.Tensor:
-        """``positions`` are not read: a row's position is its sequence's length minus the rows behind it.  ``kv_caches``:
+        """``positions`` (int64, one per row) spare the rotation a lookup of the row's sequence; without them a row's
+        position is its sequence's length minus the rows behind it, which is also what the attention's mask goes by.  ``kv_caches``:
         one page tensor per attention layer, in layer order, bound before the step (callers without an engine).
         ``residual_out``: a list that receives the sum of the streams after every layer (debugging; it splits the fused
         write-and-read launches)."""
@@ -91,7 +92,9 @@ class LidizenModel(torch.nn.Module):
         kwargs.setdefault("finished_requests_ids", [])
         (prev_token,), slot_idx = self.state_cache.current_run_tensors(**kwargs)
         input_ids = input_ids.to(torch.int64).contiguous()
-        layout = self.layout_of(md, slot_idx, input_ids)
+        if positions is not None:
+            positions = positions.to(torch.int64).contiguous()
+        layout = self.layout_of(md, slot_idx, input_ids, positions)
         big = self.config.bigram
         x = hip_ops.embed_pair(input_ids, self.embed, self.pair_table, self.embed_norm, self.config.norm_eps, self.streams,
                                buckets=big.buckets if big else 0, mul_prev=big.mul_prev if big else 0, mul_cur=big.mul_cur if big else 0,

@@ -33,6 +33,7 @@ class StepLayout:
     max_query_len: int
     max_seq_len: int
     token_ids: Optional[torch.Tensor] = None
+    positions: Optional[torch.Tensor] = None      # int64 [rows], where the caller of the model gave them
 
 
 class NormConvIn(torch.nn.Module):

@@ -87,7 +87,7 @@ class TalkingHeadsAttentionMixer(torch.nn.Module):
         other = v_first if self.blend is not None else None
         q = hip_ops.talk_qkv_prep(qkv, H, G, D, Dv, self.q_norm_weight, self.k_norm_weight, self.talk, self.eps, self.rot_dims,
                                   self.rot_freqs, attn.cache(), layout.slot_mapping, layout.query_start_loc, layout.seq_lens,
-                                  v_other=other, v_blend=self.blend if other is not None else 0.0)
+                                  v_other=other, v_blend=self.blend if other is not None else 0.0, positions=getattr(layout, "positions", None))
         if self.blend is not None and v_first is None:
             v_first = qkv[:, (H + G) * D:]
         o = attn(q, layout)
