@@ -32,7 +32,11 @@
  *    act_limit / act_alpha; the post-norm, latent- and linear-attention building blocks at the end of this file;
  *    version 6: hymeta_sink_attention_args ends with keep_first, hymeta_moe_route_sigmoid_args with router_bias /
  *    score_mode; HYMETA_KV_SHARED_KEY, HYMETA_GLU_RELU2, HYMETA_ACT_SILU_MUL / HYMETA_ACT_RELU2; the hyper-connection
- *    and talking-heads building blocks at the end of this file).
+ *    and talking-heads building blocks at the end of this file;
+ *    version 7: hymeta_sink_attention_args ends with softcap / head_gate / head_gate_stride_t, hymeta_embed_rows_args with
+ *    scale, hymeta_gated_rms_norm_args with groups / gate_act / gate_first, hymeta_moe_route_sigmoid_args with the grouped
+ *    choice's fields; HYMETA_ROUTE_SOFTMAX_GROUPED; the parallel-layer, rotate-half, state-space and decayed-scan building
+ *    blocks at the end of this file).
  *  - Every argument struct starts with `uint32_t struct_size`, which the caller
  *    sets to sizeof(the struct) of ITS declaration.  An entry point returns
  *    HYMETA_ERR_INVALID_ARG, before it reads any other field, when the value
@@ -50,7 +54,7 @@
 extern "C" {
 #endif
 
-#define HYMETA_ABI_VERSION 6
+#define HYMETA_ABI_VERSION 7
 
 typedef void* hymeta_stream_t;
 
@@ -1083,6 +1087,7 @@ typedef struct hymeta_embed_rows_args {
   const float* add;            /* [width] or NULL */
   float* out;                  /* [num_tokens, width] contiguous */
   int32_t num_tokens, width, vocab, act_dtype;
+  float scale;                 /* the rows are multiplied by it (0: by 1) before add */
 } hymeta_embed_rows_args;
 int hymeta_embed_rows(const hymeta_embed_rows_args* args, hymeta_stream_t stream);
 
@@ -1209,6 +1214,10 @@ typedef struct hymeta_sink_attention_args {
   const float* sink_logits;    /* [num_heads] or NULL: the sink's score per head (NULL: 0); read when sink != 0 */
   int32_t kv_layout;           /* enum hymeta_kv_layout */
   int32_t keep_first;          /* >= 0; read when window_left >= 0 */
+  float softcap;               /* > 0: scores (after scale, before the bias) become softcap * tanh(score / softcap) */
+  const void* head_gate;       /* act_dtype [num_tokens, num_heads], row stride head_gate_stride_t, or NULL: head h's
+                                  output of row t is multiplied by sigmoid(head_gate[t, h]) */
+  int64_t head_gate_stride_t;
 } hymeta_sink_attention_args;
 size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t num_kv_heads, int32_t v_dim,
                                              int32_t max_seq_len);
@@ -1370,7 +1379,11 @@ size_t hymeta_lightning_attention_workspace_bytes(int32_t num_seqs, int32_t num_
                                                   int32_t max_query_len);
 int hymeta_lightning_attention(const hymeta_lightning_attention_args* args, hymeta_stream_t stream);
 
-/* out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * weight * sigmoid(gate[t]): the output norm and gate of a linear attention. */
+/* out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * weight * sigmoid(gate[t]): the output norm and gate of a linear attention.
+ * groups > 1: the mean is taken over each of `groups` equal consecutive parts of the row.  gate_act: the gate's function
+ * (HYMETA_GATE_SIGMOID: sigmoid(g); HYMETA_GATE_SILU: g sigmoid(g)).  gate_first != 0: the gate multiplies x BEFORE the norm,
+ * out = norm(x * act(gate)) * weight.  weight NULL: ones. */
+enum hymeta_gate_act { HYMETA_GATE_SIGMOID = 0, HYMETA_GATE_SILU = 1 };
 typedef struct hymeta_gated_rms_norm_args {
   uint32_t struct_size;
   const float* x;              /* fp32 [num_tokens, width] contiguous */
@@ -1380,6 +1393,9 @@ typedef struct hymeta_gated_rms_norm_args {
   int32_t num_tokens, width, act_dtype;
   float eps;
   int64_t gate_stride_t;
+  int32_t groups;              /* 0 or 1: the whole row */
+  int32_t gate_act;            /* enum hymeta_gate_act */
+  int32_t gate_first;
 } hymeta_gated_rms_norm_args;
 int hymeta_gated_rms_norm(const hymeta_gated_rms_norm_args* args, hymeta_stream_t stream);
 
@@ -1408,8 +1424,16 @@ int hymeta_activation(const hymeta_activation_args* args, hymeta_stream_t stream
 /* Router of a mixture of experts: logits = x router_weight^T (+ router_bias) in fp32; the top_k largest are chosen (the
  * lower expert on a tie).  HYMETA_ROUTE_SIGMOID_SUM: s = sigmoid(logits), weights s / (sum of the chosen s + 1e-20) * scale.
  * HYMETA_ROUTE_SOFTMAX_CHOSEN: weights = softmax over the chosen logits alone, times scale.
+ * HYMETA_ROUTE_SOFTMAX_GROUPED: s = softmax(logits) over all num_experts outputs; the choice goes by s + correction;
+ * the outputs form num_groups equal runs of neighbours, a group's score is its largest corrected score, and only outputs
+ * of the keep_groups best groups can be chosen (the lower group on a tie); weights = s of the chosen (uncorrected, not
+ * renormalised) times scale.  Outputs first_identity .. num_experts - 1 are identity experts (first_identity <= 0: none):
+ * their pairs get pair_pos -1 and are left out of expert_offsets / sorted_pair (the grouped GEMMs and the combine skip
+ * them), and identity_weight[t] receives the sum of their weights -- whoever adds the block's output adds identity_weight[t]
+ * times the block's input.  extra_rows (0 or 1): router_weight holds that many more rows behind the num_experts router
+ * rows; sigmoid of row num_experts' product goes to extra_out[t] (a gate of one number per token computed alongside).
  * Writes what hymeta_moe_route writes.  num_experts <= HYMETA_MOE_TABLE_MAX_EXPERTS. */
-enum hymeta_route_mode { HYMETA_ROUTE_SIGMOID_SUM = 0, HYMETA_ROUTE_SOFTMAX_CHOSEN = 1 };
+enum hymeta_route_mode { HYMETA_ROUTE_SIGMOID_SUM = 0, HYMETA_ROUTE_SOFTMAX_CHOSEN = 1, HYMETA_ROUTE_SOFTMAX_GROUPED = 2 };
 typedef struct hymeta_moe_route_sigmoid_args {
   uint32_t struct_size;
   const void* x;               /* act_dtype [num_tokens, hidden], row stride x_stride_t */
@@ -1424,6 +1448,11 @@ typedef struct hymeta_moe_route_sigmoid_args {
   int64_t x_stride_t;
   const float* router_bias;    /* [num_experts] or NULL */
   int32_t score_mode;          /* enum hymeta_route_mode */
+  /* HYMETA_ROUTE_SOFTMAX_GROUPED */
+  int32_t num_groups, keep_groups, first_identity, extra_rows;
+  const float* correction;     /* [num_experts] or NULL */
+  float* identity_weight;      /* out [num_tokens]; required when first_identity > 0 */
+  float* extra_out;            /* out [num_tokens]; required when extra_rows > 0 */
 } hymeta_moe_route_sigmoid_args;
 int hymeta_moe_route_sigmoid(const hymeta_moe_route_sigmoid_args* args, hymeta_stream_t stream);
 
@@ -1504,6 +1533,109 @@ typedef struct hymeta_talk_qkv_prep_args {
   const int64_t* positions;    /* [num_tokens] or NULL: a row's position is its sequence's length minus the rows behind it */
 } hymeta_talk_qkv_prep_args;
 int hymeta_talk_qkv_prep(const hymeta_talk_qkv_prep_args* args, hymeta_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Building blocks of parallel-layer designs (one norm, mixer and feed-forward side by side) with rotate-half rotary
+ * attention, retention, and state-space (Mamba-2) mixers.
+ * ---------------------------------------------------------------------- */
+
+/* x[t] += sum_i coef[i] * (row_scale[i] ? row_scale[i][t] : 1) * y[i][t] on the fp32 stream, in place (fp32 sums, terms
+ * added in order); then, with h_out, h_out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * norm_scale (ONE number for all columns;
+ * norm_weight, if given, also multiplies per column) rounded to act_dtype: a parallel layer's sum and the next layer's
+ * norm in one launch.  num_terms = 0: the norm alone. */
+#define HYMETA_STREAM_MAX_TERMS 6
+typedef struct hymeta_stream_add_norm_args {
+  uint32_t struct_size;
+  float* x;                    /* [num_tokens, width], row stride x_stride_t */
+  const void* y[HYMETA_STREAM_MAX_TERMS];           /* act_dtype [num_tokens, width], row stride y_stride_t[i] */
+  const float* row_scale[HYMETA_STREAM_MAX_TERMS];  /* [num_tokens] or NULL */
+  float coef[HYMETA_STREAM_MAX_TERMS];
+  int64_t y_stride_t[HYMETA_STREAM_MAX_TERMS];
+  const float* norm_weight;    /* [width] or NULL */
+  void* h_out;                 /* act_dtype [num_tokens, width] contiguous, or NULL */
+  int32_t num_tokens, width, num_terms, act_dtype;
+  float eps, norm_scale;
+  int64_t x_stride_t;
+} hymeta_stream_add_norm_args;
+int hymeta_stream_add_norm(const hymeta_stream_add_norm_args* args, hymeta_stream_t stream);
+
+/* Between a fused q | k | v (| ...) projection and an attention or a recurrence, per token, one launch, in place:
+ *   of the first rot_dims dimensions of every query and key head, i and i + rot_dims / 2 turn together by
+ *   position * rot_freqs[i] ("rotate half": (u, v) -> (u cos - v sin, v cos + u sin)); the rest pass; angles are reduced in
+ *   double precision, the turn is fp32;
+ *   keys are then multiplied by k_scale (0: by 1);
+ *   with kv_cache: the cache row at slot_mapping[t] <- per key/value head the key followed by the value
+ *   (HYMETA_KV_KEY_THEN_VALUE, as hymeta_sink_attention reads it).
+ * A row's position is positions[t], or without positions its sequence's length minus the rows behind it. */
+typedef struct hymeta_rotary_cache_args {
+  uint32_t struct_size;
+  void* qkv;                   /* act_dtype [num_tokens, H D + G D + G Dv (+ more)], row stride qkv_stride_t */
+  const double* rot_freqs;     /* [rot_dims / 2] or NULL when rot_dims == 0 */
+  void* kv_cache;              /* act_dtype [blocks, block_size, G, D + Dv] or NULL */
+  const int64_t* slot_mapping; /* [num_tokens] or NULL */
+  const int64_t* positions;    /* [num_tokens] or NULL */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] (without positions) */
+  const int32_t* seq_lens;         /* [num_seqs] (without positions) */
+  int32_t num_tokens, num_seqs, num_heads, num_kv_heads, head_dim, v_dim, rot_dims, block_size, act_dtype;
+  float k_scale;
+  int64_t num_blocks, qkv_stride_t;
+} hymeta_rotary_cache_args;
+int hymeta_rotary_cache(const hymeta_rotary_cache_args* args, hymeta_stream_t stream);
+
+/* Short causal convolution over time per channel with bias and silu, over each sequence's rows, and the step sizes of
+ * a state-space layer, one launch:
+ *   out[t, c] = silu(bias[c] + sum_{j < taps} weight[c, j] * x[t - (taps - 1) + j, c])     (zeros before a sequence's start)
+ *   dt[t, h]  = softplus(dt_in[t, h] + dt_bias[h])                                          (fp32, no clamp)
+ *   log2_decay[t, h] = -exp(a_log[h]) * dt[t, h] * log2(e)                                  (fp32)
+ * conv_state [slots, taps - 1, channels] (act_dtype) holds a sequence's last taps - 1 INPUT rows between steps: read
+ * where context_lens > 0, rewritten by a second launch.  dt_in NULL: the convolution alone.  taps <= HYMETA_CONV_MAX_TAPS. */
+typedef struct hymeta_causal_conv_args {
+  uint32_t struct_size;
+  const void* x;               /* act_dtype [num_tokens, channels], row stride x_stride_t */
+  const float* weight;         /* [channels, taps] */
+  const float* bias;           /* [channels] or NULL */
+  void* out;                   /* act_dtype [num_tokens, channels] contiguous */
+  void* conv_state;            /* act_dtype [slots, taps - 1, channels] or NULL */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] */
+  const int32_t* context_lens;     /* [num_seqs] */
+  const int32_t* slot_idx;         /* [num_seqs] */
+  const void* dt_in;           /* act_dtype [num_tokens, dt_heads], row stride dt_stride_t; or NULL */
+  const float* dt_bias;        /* [dt_heads] */
+  const float* a_log;          /* [dt_heads] */
+  float* dt_out;               /* [num_tokens, dt_heads] */
+  float* log2_decay_out;       /* [num_tokens, dt_heads] */
+  int32_t num_tokens, num_seqs, channels, taps, dt_heads, act_dtype;
+  int64_t x_stride_t, dt_stride_t;
+} hymeta_causal_conv_args;
+int hymeta_causal_conv(const hymeta_causal_conv_args* args, hymeta_stream_t stream);
+
+/* Linear recurrence with a scalar decay per head and token over a step's rows, the state fp32 [slots, H, D, Dv]:
+ *   S_t = a_t S_{t-1} + b_t k_t v_t^T,   out_t = S_t^T q_t + skip[h] v_t
+ * a_t = exp2(log2_decay[t, h]) per token, or decay[h] for all tokens (log2_decay NULL); b_t = v_scale[t, h] or 1;
+ * query / key head of head h: h / (num_heads / num_qk_heads) (one q and k per group of heads).  This is retention
+ * (constant decay, no skip) and the state-space duality form of Mamba-2 (q = C, k = B, v = x, b = dt).  Inputs enter as
+ * they are (no activation).  Rows of sequences with one row run a step kernel, bf16 portions of
+ * HYMETA_SCAN_CHUNK-row chunks on the matrix cores (head_dim 32 / 64 / 128, v_dim in whole 32s), everything else token by
+ * token.  The state is read where context_lens > 0 and written. */
+#define HYMETA_SCAN_CHUNK 64
+typedef struct hymeta_decay_scan_args {
+  uint32_t struct_size;
+  const void* q;               /* act_dtype [num_tokens, num_qk_heads, head_dim], row stride q_stride_t */
+  const void* k;               /* likewise, row stride k_stride_t */
+  const void* v;               /* act_dtype [num_tokens, num_heads, v_dim], row stride v_stride_t */
+  float* state;
+  const float* decay;          /* [num_heads] (log2_decay NULL) */
+  const float* log2_decay;     /* [num_tokens, num_heads] or NULL */
+  const float* v_scale;        /* [num_tokens, num_heads] or NULL */
+  const float* skip;           /* [num_heads] or NULL */
+  float* out;                  /* fp32 [num_tokens, num_heads * v_dim] contiguous */
+  const int32_t* query_start_loc;
+  const int32_t* context_lens;
+  const int32_t* slot_idx;
+  int32_t num_tokens, num_seqs, num_heads, num_qk_heads, head_dim, v_dim, act_dtype, max_query_len;
+  int64_t q_stride_t, k_stride_t, v_stride_t;
+} hymeta_decay_scan_args;
+int hymeta_decay_scan(const hymeta_decay_scan_args* args, hymeta_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -58,37 +58,49 @@ __global__ __launch_bounds__(256) void lightning_rows_kernel(hymeta_lightning_at
 // Rows of up to kGatedCached columns are read once (a thread keeps its columns in registers).
 constexpr int kGatedPerThread = 16, kGatedCached = 256 * kGatedPerThread;
 
+// grid = (rows, groups): a workgroup norms one of the row's equal consecutive parts.
 template <typename A, bool Cached>
 __global__ __launch_bounds__(256) void gated_rms_norm_kernel(hymeta_gated_rms_norm_args a) {
   typedef typename A::elem elem;
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
-  const float* x = a.x + t * a.width;
-  const elem* g = static_cast<const elem*>(a.gate) + t * a.gate_stride_t;
-  elem* out = static_cast<elem*>(a.out) + t * a.width;
+  const int width = a.width / gridDim.y, c0 = blockIdx.y * width;
+  const float* x = a.x + t * a.width + c0;
+  const elem* g = static_cast<const elem*>(a.gate) + t * a.gate_stride_t + c0;
+  const float* weight = a.weight ? a.weight + c0 : nullptr;
+  elem* out = static_cast<elem*>(a.out) + t * a.width + c0;
+  const bool silu = a.gate_act == HYMETA_GATE_SILU, first = a.gate_first != 0;
+  auto gate_of = [&](float gv) { const float sg = sigmoid_exact(gv); return silu ? gv * sg : sg; };
   float ss = 0.f;
   if (Cached) {
     float xv[kGatedPerThread], gv[kGatedPerThread];
 #pragma unroll
     for (int u = 0; u < kGatedPerThread; ++u) {
       const int c = threadIdx.x + 256 * u;
-      xv[u] = c < a.width ? x[c] : 0.f;
-      gv[u] = c < a.width ? A::ld(g + c) : 0.f;
+      xv[u] = c < width ? x[c] : 0.f;
+      gv[u] = c < width ? gate_of(A::ld(g + c)) : 0.f;
+      if (first) xv[u] *= gv[u], gv[u] = 1.f;
       ss = fmaf(xv[u], xv[u], ss);
     }
     ss = block_sum<4>(ss, red);
-    const float inv = 1.f / sqrtf(ss / static_cast<float>(a.width) + a.eps);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(width) + a.eps);
 #pragma unroll
     for (int u = 0; u < kGatedPerThread; ++u) {
       const int c = threadIdx.x + 256 * u;
-      if (c < a.width) A::st(out + c, xv[u] * inv * a.weight[c] * sigmoid_exact(gv[u]));
+      if (c < width) A::st(out + c, xv[u] * inv * (weight ? weight[c] : 1.f) * gv[u]);
     }
     return;
   }
-  for (int c = threadIdx.x; c < a.width; c += 256) ss = fmaf(x[c], x[c], ss);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = first ? x[c] * gate_of(A::ld(g + c)) : x[c];
+    ss = fmaf(v, v, ss);
+  }
   ss = block_sum<4>(ss, red);
-  const float inv = 1.f / sqrtf(ss / static_cast<float>(a.width) + a.eps);
-  for (int c = threadIdx.x; c < a.width; c += 256) A::st(out + c, x[c] * inv * a.weight[c] * sigmoid_exact(A::ld(g + c)));
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(width) + a.eps);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float gv = gate_of(A::ld(g + c));
+    A::st(out + c, x[c] * inv * (weight ? weight[c] : 1.f) * gv);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -494,15 +506,18 @@ extern "C" int hymeta_gated_rms_norm(const hymeta_gated_rms_norm_args* args, hym
   if (a.num_tokens < 0 || a.width <= 0) return HYMETA_ERR_INVALID_ARG;
   if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
   if (a.num_tokens == 0) return HYMETA_OK;
-  if (!a.x || !a.gate || !a.weight || !a.out || a.gate_stride_t < a.width) return HYMETA_ERR_INVALID_ARG;
+  if (!a.x || !a.gate || !a.out || a.gate_stride_t < a.width) return HYMETA_ERR_INVALID_ARG;
+  const int groups = a.groups > 1 ? a.groups : 1;
+  if (a.width % groups != 0 || groups > 65535) return HYMETA_ERR_INVALID_ARG;
+  if (a.gate_act != HYMETA_GATE_SIGMOID && a.gate_act != HYMETA_GATE_SILU) return HYMETA_ERR_UNSUPPORTED;
   hipStream_t st = begin_launches(stream);
-  const bool cached = a.width <= kGatedCached;
+  const bool cached = a.width / groups <= kGatedCached;
   if (a.act_dtype == HYMETA_BF16) {
-    if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, true>), dim3(a.num_tokens), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, false>), dim3(a.num_tokens), dim3(256), 0, st, a);
+    if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, true>), dim3(a.num_tokens, groups), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, false>), dim3(a.num_tokens, groups), dim3(256), 0, st, a);
   } else {
-    if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActF32, true>), dim3(a.num_tokens), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gated_rms_norm_kernel<ActF32, false>), dim3(a.num_tokens), dim3(256), 0, st, a);
+    if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActF32, true>), dim3(a.num_tokens, groups), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gated_rms_norm_kernel<ActF32, false>), dim3(a.num_tokens, groups), dim3(256), 0, st, a);
   }
   return launch_status();
 }

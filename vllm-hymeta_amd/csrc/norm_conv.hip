@@ -22,7 +22,8 @@ __global__ __launch_bounds__(kNormThreads) void embed_rows_kernel(hymeta_embed_r
   if (tok < 0 || tok >= a.vocab) tok = 0;          // ids are validated on the host; never read out of the table
   const typename A::elem* row = static_cast<const typename A::elem*>(a.table) + tok * a.width;
   float* out = a.out + static_cast<int64_t>(t) * a.width;
-  for (int c = threadIdx.x; c < a.width; c += kNormThreads) out[c] = A::ld(row + c) + (a.add ? a.add[c] : 0.f);
+  const float scale = a.scale != 0.f ? a.scale : 1.f;
+  for (int c = threadIdx.x; c < a.width; c += kNormThreads) out[c] = A::ld(row + c) * scale + (a.add ? a.add[c] : 0.f);
 }
 
 __device__ __forceinline__ int seq_of_row_fast(const hymeta_norm_conv_args& a, int t);

@@ -106,7 +106,9 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
         const elem* k = cache + roff + key_off;
         float dot = 0.f;
         for (int d = 0; d < D; ++d) dot = fmaf(s_q[d], A::ld(k + d), dot);
-        sc = dot * a.scale - distance_bias(a.bias_mode, ba, bb, pos - j);
+        sc = dot * a.scale;
+        if (a.softcap > 0.f) sc = a.softcap * tanhf(sc / a.softcap);
+        sc -= distance_bias(a.bias_mode, ba, bb, pos - j);
       }
       const float m_new = fmaxf(m, wave_max(sc));
       const float p = valid ? expf(sc - m_new) : 0.f;
@@ -131,7 +133,8 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
     }
   }
   elem* out = static_cast<elem*>(a.out) + (static_cast<int64_t>(t) * a.num_heads + h) * Dv;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float inv = l > 0.f ? 1.f / l : 0.f;
+  if (a.head_gate) inv *= sigmoid_exact(A::ld(static_cast<const elem*>(a.head_gate) + static_cast<int64_t>(t) * a.head_gate_stride_t + h));
 #pragma unroll
   for (int cc = 0; cc < kMaxVChunks; ++cc) {
     const int c = cc * 64 + lane;
@@ -305,6 +308,11 @@ struct WaveRows {
 
 typedef short bf16x4 __attribute__((ext_vector_type(4)));
 
+// tanh through the hardware's exponential: 1 - 2 / (exp(2 x) + 1), exact at both ends (exp2 -> inf gives 1, -> 0 gives -1)
+__device__ __forceinline__ float tanh_fast(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
+}
+
 template <int D, int DV, int RB, int NKS, bool Masked>
 __device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a,
                                             int j0, int ks_lo) {
@@ -330,6 +338,9 @@ __device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSm
   // maximum, and with it the sink's score 0, mean the same in both domains.
   const float scale2 = a.scale * 1.4426950408889634f;
   const bool bias = a.bias_mode == HYMETA_BIAS_LOG_DISTANCE;
+  // capped scores: softcap tanh(score / softcap), moved into the base-2 domain like the others
+  const bool capped = a.softcap > 0.f;
+  const float cap2 = a.softcap * 1.4426950408889634f, cap_in = capped ? a.scale / a.softcap : 0.f;
   uint32_t phi[RB][NKS][2], plo[RB][NKS][2];       // the weights' bf16 high and low parts, two per dword
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -342,6 +353,7 @@ __device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSm
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float sc = s[rb][ks][r] * scale2;
+        if (capped) sc = cap2 * tanh_fast(s[rb][ks][r] * cap_in);
         if (bias) sc = fmaf(-w.ba[rb], __log2f(fmaf(w.bb[rb], fd0 - static_cast<float>(16 * ks + r), 1.f)), sc);
         if (Masked) {
           const int j = j0 + 16 * (ks_lo + ks) + 4 * g4 + r;
@@ -508,7 +520,8 @@ __global__ __launch_bounds__(64 * PrefillWaves<D>::value) void sink_attention_pr
     l += __shfl_xor(l, 32, 64);
     const int r = wrow + 16 * rb + n;
     if (r >= q) continue;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float inv = l > 0.f ? 1.f / l : 0.f;
+    if (a.head_gate) inv *= sigmoid_exact(bf2f(static_cast<const uint16_t*>(a.head_gate)[static_cast<int64_t>(row0 + r) * a.head_gate_stride_t + h]));
     uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(row0 + r) * a.num_heads + h) * vs.total + vs.first;
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb) {
@@ -704,7 +717,8 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
     const float ms = base[sp * stride + DV];
     if (ms != -INFINITY) l += base[sp * stride + DV + 1] * __builtin_amdgcn_exp2f(ms - m);
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float inv = l > 0.f ? 1.f / l : 0.f;
+  if (a.head_gate) inv *= sigmoid_exact(bf2f(static_cast<const uint16_t*>(a.head_gate)[static_cast<int64_t>(t) * a.head_gate_stride_t + h]));
   uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(t) * a.num_heads + h) * vs.total + vs.first;
   for (int c = threadIdx.x; c < DV; c += 64) {
     float acc = 0.f;
@@ -821,6 +835,7 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
   if (a.num_tokens == 0 || a.num_seqs == 0) return HYMETA_OK;
   if (!a.q || !a.kv_cache || !a.out || !a.block_tables || !a.query_start_loc || !a.seq_lens) return HYMETA_ERR_INVALID_ARG;
   if (a.bias_mode != HYMETA_BIAS_NONE && (!a.bias_a || !a.bias_b)) return HYMETA_ERR_INVALID_ARG;
+  if (a.softcap < 0.f || (a.head_gate && a.head_gate_stride_t < a.num_heads)) return HYMETA_ERR_INVALID_ARG;
   if (a.num_heads > 65535) return HYMETA_ERR_UNSUPPORTED;
   hipStream_t st = begin_launches(stream);
   if (mfma_shape(a) && a.max_query_len >= 1 && a.max_seq_len >= 1) {

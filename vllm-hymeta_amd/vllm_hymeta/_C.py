@@ -31,12 +31,15 @@ KV_VALUE_IN_KEY = 1
 KV_SHARED_KEY = 2
 GLU_NONE, GLU_SILU, GLU_CLAMPED, GLU_RELU2 = 0, 1, 2, 3
 ACT_CLAMPED_GLU, ACT_XIELU, ACT_SIGMOID_MUL, ACT_SILU_MUL, ACT_RELU2 = 0, 1, 2, 3, 4
-ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN = 0, 1
+ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN, ROUTE_SOFTMAX_GROUPED = 0, 1, 2
+GATE_SIGMOID, GATE_SILU = 0, 1
+STREAM_MAX_TERMS = 6
+SCAN_CHUNK = 64
 MAX_STREAMS = 16
 LIGHTNING_CHUNK = 64
 CONV_MAX_TAPS = 8
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 ERR_SCRATCH_LIMIT = -5
 GEMM_TICKET_BYTES = 16384
 STATIC_SCRATCH_BYTES = 16 << 20
@@ -304,6 +307,7 @@ class EmbedRowsArgs(_Args):
         _SIZE,
         ("token_ids", _ptr), ("table", _ptr), ("add", _ptr), ("out", _ptr),
         ("num_tokens", _i32), ("width", _i32), ("vocab", _i32), ("act_dtype", _i32),
+        ("scale", _f32),
     ]
 
 
@@ -360,6 +364,7 @@ class SinkAttentionArgs(_Args):
         ("scale", _f32),
         ("num_blocks", _i64), ("q_stride_t", _i64), ("block_table_stride", _i64),
         ("sink_logits", _ptr), ("kv_layout", _i32), ("keep_first", _i32),
+        ("softcap", _f32), ("head_gate", _ptr), ("head_gate_stride_t", _i64),
     ]
 
 
@@ -454,6 +459,7 @@ class GatedRmsNormArgs(_Args):
         ("num_tokens", _i32), ("width", _i32), ("act_dtype", _i32),
         ("eps", _f32),
         ("gate_stride_t", _i64),
+        ("groups", _i32), ("gate_act", _i32), ("gate_first", _i32),
     ]
 
 
@@ -476,6 +482,8 @@ class MoeRouteSigmoidArgs(_Args):
         ("scale", _f32),
         ("x_stride_t", _i64),
         ("router_bias", _ptr), ("score_mode", _i32),
+        ("num_groups", _i32), ("keep_groups", _i32), ("first_identity", _i32), ("extra_rows", _i32),
+        ("correction", _ptr), ("identity_weight", _ptr), ("extra_out", _ptr),
     ]
 
 
@@ -510,6 +518,52 @@ class TalkQkvPrepArgs(_Args):
         ("eps", _f32), ("v_blend", _f32),
         ("num_blocks", _i64), ("qkv_stride_t", _i64), ("v_other_stride_t", _i64),
         ("positions", _ptr),
+    ]
+
+
+
+class StreamAddNormArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("y", _ptr * STREAM_MAX_TERMS), ("row_scale", _ptr * STREAM_MAX_TERMS), ("coef", _f32 * STREAM_MAX_TERMS),
+        ("y_stride_t", _i64 * STREAM_MAX_TERMS), ("norm_weight", _ptr), ("h_out", _ptr),
+        ("num_tokens", _i32), ("width", _i32), ("num_terms", _i32), ("act_dtype", _i32),
+        ("eps", _f32), ("norm_scale", _f32),
+        ("x_stride_t", _i64),
+    ]
+
+
+class RotaryCacheArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("qkv", _ptr), ("rot_freqs", _ptr), ("kv_cache", _ptr), ("slot_mapping", _ptr), ("positions", _ptr),
+        ("query_start_loc", _ptr), ("seq_lens", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32), ("v_dim", _i32),
+        ("rot_dims", _i32), ("block_size", _i32), ("act_dtype", _i32),
+        ("k_scale", _f32),
+        ("num_blocks", _i64), ("qkv_stride_t", _i64),
+    ]
+
+
+class CausalConvArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("weight", _ptr), ("bias", _ptr), ("out", _ptr), ("conv_state", _ptr),
+        ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("dt_in", _ptr), ("dt_bias", _ptr), ("a_log", _ptr), ("dt_out", _ptr), ("log2_decay_out", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("channels", _i32), ("taps", _i32), ("dt_heads", _i32), ("act_dtype", _i32),
+        ("x_stride_t", _i64), ("dt_stride_t", _i64),
+    ]
+
+
+class DecayScanArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("q", _ptr), ("k", _ptr), ("v", _ptr), ("state", _ptr), ("decay", _ptr), ("log2_decay", _ptr), ("v_scale", _ptr),
+        ("skip", _ptr), ("out", _ptr), ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("num_qk_heads", _i32), ("head_dim", _i32), ("v_dim", _i32),
+        ("act_dtype", _i32), ("max_query_len", _i32),
+        ("q_stride_t", _i64), ("k_stride_t", _i64), ("v_stride_t", _i64),
     ]
 
 
@@ -603,6 +657,10 @@ _SIGNATURES = {
     "hymeta_embed_pair": (C.c_int, [C.POINTER(EmbedPairArgs), _ptr]),
     "hymeta_hyper_stream": (C.c_int, [C.POINTER(HyperStreamArgs), _ptr]),
     "hymeta_talk_qkv_prep": (C.c_int, [C.POINTER(TalkQkvPrepArgs), _ptr]),
+    "hymeta_stream_add_norm": (C.c_int, [C.POINTER(StreamAddNormArgs), _ptr]),
+    "hymeta_rotary_cache": (C.c_int, [C.POINTER(RotaryCacheArgs), _ptr]),
+    "hymeta_causal_conv": (C.c_int, [C.POINTER(CausalConvArgs), _ptr]),
+    "hymeta_decay_scan": (C.c_int, [C.POINTER(DecayScanArgs), _ptr]),
 }
 
 STRUCTS = {
@@ -644,6 +702,10 @@ STRUCTS = {
     "hymeta_embed_pair_args": EmbedPairArgs,
     "hymeta_hyper_stream_args": HyperStreamArgs,
     "hymeta_talk_qkv_prep_args": TalkQkvPrepArgs,
+    "hymeta_stream_add_norm_args": StreamAddNormArgs,
+    "hymeta_rotary_cache_args": RotaryCacheArgs,
+    "hymeta_causal_conv_args": CausalConvArgs,
+    "hymeta_decay_scan_args": DecayScanArgs,
 }
 
 

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
-from typing import NamedTuple, Optional
+from typing import NamedTuple, Optional, Sequence, Tuple
 
 import torch
 
@@ -1476,8 +1476,8 @@ def _i32vec(t: torch.Tensor, n: int, name: str) -> None:
     _require(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n, f"{name} must be contiguous int32 [{n}]")
 
 
-def embed_rows(token_ids: torch.Tensor, table: torch.Tensor, add: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """fp32 ``[T, W]`` rows ``table[token_ids] (+ add)``: the start of an fp32 residual stream."""
+def embed_rows(token_ids: torch.Tensor, table: torch.Tensor, add: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """fp32 ``[T, W]`` rows ``table[token_ids] * scale (+ add)``: the start of an fp32 residual stream."""
     _dev(token_ids, table, add)
     _require(token_ids.dtype == torch.int64 and token_ids.dim() == 1 and token_ids.is_contiguous(), "token_ids must be contiguous int64 [T]")
     _require(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [vocab, width]")
@@ -1486,7 +1486,7 @@ def embed_rows(token_ids: torch.Tensor, table: torch.Tensor, add: Optional[torch
     out = torch.empty(token_ids.shape[0], W, dtype=torch.float32, device=table.device)
     a = _C.EmbedRowsArgs()
     a.token_ids, a.table, a.add, a.out = _p(token_ids), _p(table), _p(add), _p(out)
-    a.num_tokens, a.width, a.vocab, a.act_dtype = token_ids.shape[0], W, V, _act(table)
+    a.num_tokens, a.width, a.vocab, a.act_dtype, a.scale = token_ids.shape[0], W, V, _act(table), float(scale)
     _C.check(_C.load().hymeta_embed_rows(C.byref(a), _stream(table)), "hymeta_embed_rows")
     return out
 
@@ -1601,10 +1601,11 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
                    max_query_len: int, max_seq_len: int, bias_a: Optional[torch.Tensor] = None,
                    bias_b: Optional[torch.Tensor] = None, sink: bool = True, window_left: int = -1,
                    sink_logits: Optional[torch.Tensor] = None, value_in_key: bool = False, shared_key: bool = False,
-                   keep_first: int = 0) -> torch.Tensor:
+                   keep_first: int = 0, softcap: float = 0.0, head_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of the rows ``q [T, H, D]`` over their sequences' paged keys (this step's included):
     ``softmax`` over ``scale q.k - bias_a[h] ln(1 + bias_b[h] (i - j))`` with, for ``sink``, ``exp(sink_logits[h])`` (one
-    without ``sink_logits``) added to the denominator.  ``value_in_key``: a cache row holds ``D`` elements per key/value
+    without ``sink_logits``) added to the denominator.  ``softcap > 0``: ``scale q.k`` becomes ``softcap tanh(scale q.k /
+    softcap)``.  ``head_gate [T, H]`` (a view with any row stride): head ``h``'s output is multiplied by its sigmoid.  ``value_in_key``: a cache row holds ``D`` elements per key/value
     head, the first ``Dv`` of which are also the value (a latent that keys and values share).  Returns ``[T, H, Dv]``."""
     _dev(q, kv_cache, block_tables, query_start_loc, seq_lens, bias_a, bias_b, sink_logits)
     _require(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == head_dim and q.shape[2] == head_dim, "q must be [T, H, D] with contiguous heads")
@@ -1638,7 +1639,11 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
     a.block_size, a.act_dtype, a.num_blocks = kv_cache.shape[1], _act(q), kv_cache.shape[0]
     a.bias_mode = _C.BIAS_NONE if bias_a is None else _C.BIAS_LOG_DISTANCE
     a.sink, a.window_left, a.max_query_len, a.max_seq_len, a.scale = int(bool(sink)), window_left, max_query_len, max_seq_len, scale
-    a.sink_logits, a.keep_first = _p(sink_logits), keep_first
+    a.sink_logits, a.keep_first, a.softcap = _p(sink_logits), keep_first, float(softcap)
+    if head_gate is not None:
+        _dev(q, head_gate)
+        _require(head_gate.shape == (T, H) and head_gate.stride(1) == 1 and head_gate.dtype == q.dtype, "head_gate must be [T, H] of q's type with contiguous heads")
+        a.head_gate, a.head_gate_stride_t = _p(head_gate), head_gate.stride(0)
     a.kv_layout = _C.KV_SHARED_KEY if shared_key else (_C.KV_VALUE_IN_KEY if value_in_key else _C.KV_KEY_THEN_VALUE)
     a.q_stride_t, a.block_table_stride = q.stride(0), block_tables.stride(0)
     _C.check(lib.hymeta_sink_attention(C.byref(a), _stream(q)), "hymeta_sink_attention")
@@ -1705,7 +1710,7 @@ def moe_table_forward(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Ten
         c.num_tokens, c.hidden, c.top_k = T, H, top
         c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
         _C.check(lib.hymeta_moe_combine(C.byref(c), st), "hymeta_moe_combine")
-        return out
+        return result(out)
 
     act = _DT[x.dtype]
     hact = torch.empty(P, inter, dtype=x.dtype, device=dev)
@@ -1870,9 +1875,14 @@ def lightning_attention(qkv: torch.Tensor, state: torch.Tensor, decay: torch.Ten
     return out
 
 
-def gated_rms_norm(x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+def gated_rms_norm(x: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int = 1,
+                   gate_act: str = "sigmoid", gate_first: bool = False) -> torch.Tensor:
     """``rmsnorm(x) * weight * sigmoid(gate)``: fp32 rows ``x [T, W]``, ``gate [T, W]`` in the activations' type, which
-    is also the result's."""
+    is also the result's.  ``groups``: the root mean square is taken over each of that many equal consecutive parts of a row
+    (per head, for instance).  ``gate_act``: ``"sigmoid"`` or ``"silu"``.  ``gate_first``: the gate multiplies ``x`` before
+    the norm, ``rmsnorm(x * act(gate)) * weight``.  ``weight`` None: ones."""
+    _require(gate_act in ("sigmoid", "silu"), "gate_act is sigmoid or silu")
+    _require(groups >= 1 and x.shape[1] % groups == 0, "the width must split into equal groups")
     _dev(x, gate, weight)
     _require(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous fp32 [T, W]")
     T, W = x.shape
@@ -1882,6 +1892,7 @@ def gated_rms_norm(x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, ep
     a = _C.GatedRmsNormArgs()
     a.x, a.gate, a.weight, a.out = _p(x), _p(gate), _p(weight), _p(out)
     a.num_tokens, a.width, a.act_dtype, a.eps, a.gate_stride_t = T, W, _act(gate), eps, gate.stride(0)
+    a.groups, a.gate_act, a.gate_first = groups, (_C.GATE_SILU if gate_act == "silu" else _C.GATE_SIGMOID), int(bool(gate_first))
     _C.check(_C.load().hymeta_gated_rms_norm(C.byref(a), _stream(x)), "hymeta_gated_rms_norm")
     return out
 
@@ -1921,7 +1932,19 @@ def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
     return _activation(_C.ACT_SIGMOID_MUL, x, x.shape[1], 0.0, 0.0, gate=gate)
 
 
-ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN = _C.ROUTE_SIGMOID_SUM, _C.ROUTE_SOFTMAX_CHOSEN
+ROUTE_SIGMOID_SUM, ROUTE_SOFTMAX_CHOSEN, ROUTE_SOFTMAX_GROUPED = _C.ROUTE_SIGMOID_SUM, _C.ROUTE_SOFTMAX_CHOSEN, _C.ROUTE_SOFTMAX_GROUPED
+
+
+class GroupedChoice(NamedTuple):
+    """What ``ROUTE_SOFTMAX_GROUPED`` needs beside the router's matrix: ``correction [outputs]`` added to the scores for the
+    choice alone (None: nothing), ``groups`` equal runs of neighbouring outputs of which the ``keep`` best can be chosen
+    from, the last ``identity`` outputs being identity experts, and ``extra_rows`` (0 or 1) more rows behind the router's
+    whose sigmoid comes back as a gate of one number per token."""
+    correction: Optional[torch.Tensor]
+    groups: int = 1
+    keep: int = 1
+    identity: int = 0
+    extra_rows: int = 0
 
 
 def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, top_k: int,
@@ -1935,30 +1958,44 @@ def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch
 
 def moe_routed_forward(x: torch.Tensor, router_weight: torch.Tensor, router_bias: Optional[torch.Tensor], w1: torch.Tensor,
                        w2: torch.Tensor, top_k: int, score_mode: int, route_scale: float, expert_act: str, limit: float = 0.0,
-                       alpha: float = 1.702) -> torch.Tensor:
+                       alpha: float = 1.702, choice: Optional[GroupedChoice] = None):
     """Experts chosen by the ``top_k`` largest router logits ``x router_weight^T (+ router_bias)`` (fp32; the lower expert
-    on a tie).  ``score_mode``: ``ROUTE_SIGMOID_SUM`` (weights = sigmoid scores over the chosen's sum) or
-    ``ROUTE_SOFTMAX_CHOSEN`` (softmax over the chosen logits alone), times ``route_scale``.  ``expert_act``:
-    ``"clamped_glu"``: ``w1 [E, 2I, H]`` (gate rows, then up rows), ``g sigmoid(alpha g) (u + 1)`` clamped at ``limit``;
-    ``"relu2"``: ``w1 [E, I, H]``, ``max(z, 0)^2``.  ``w2 [E, H, I]``; all bf16 or all fp32.  bf16 experts in the MFMA
-    tiles' shapes run the routed block's grouped GEMMs, everything else the generic grouped GEMM with the activation in its
-    epilogue."""
+    on a tie).  ``score_mode``: ``ROUTE_SIGMOID_SUM`` (weights = sigmoid scores over the chosen's sum),
+    ``ROUTE_SOFTMAX_CHOSEN`` (softmax over the chosen logits alone) or ``ROUTE_SOFTMAX_GROUPED`` (softmax over all outputs,
+    the choice by corrected scores within the best groups, identity experts: ``choice``), times ``route_scale``.
+    ``expert_act``: ``"clamped_glu"``: ``w1 [E, 2I, H]`` (gate rows, then up rows), ``g sigmoid(alpha g) (u + 1)`` clamped at
+    ``limit``; ``"silu_glu"``: the same rows, ``silu(g) u``; ``"relu2"``: ``w1 [E, I, H]``, ``max(z, 0)^2``.  ``w2 [E, H, I]``;
+    all bf16 or all fp32.  bf16 experts in the MFMA tiles' shapes run the routed block's grouped GEMMs, everything else the
+    generic grouped GEMM with the activation in its epilogue.  With ``choice`` the result is ``(out, identity_weight [T] or
+    None, gate [T] or None)``: ``out`` holds the real experts' sum; the caller adds ``identity_weight[t] * x[t]``."""
     _dev(x, router_weight, router_bias, w1, w2)
-    _require(expert_act in ("clamped_glu", "relu2"), "expert_act is clamped_glu or relu2")
-    gated = expert_act == "clamped_glu"
+    _require(expert_act in ("clamped_glu", "silu_glu", "relu2"), "expert_act is clamped_glu, silu_glu or relu2")
+    _require((score_mode == _C.ROUTE_SOFTMAX_GROUPED) == (choice is not None), "the grouped choice comes with its constants")
+    gated = expert_act != "relu2"
     T, H = x.shape
     E, n1, _ = w1.shape
+    outputs = E if choice is None else E + choice.identity           # the router's outputs that enter the softmax
+    rows = outputs if choice is None else outputs + choice.extra_rows
     inter = n1 // 2 if gated else n1
     _require(x.dtype in _DT and x.stride(1) == 1 and w1.dtype == x.dtype and w2.dtype == x.dtype, "x, w1 and w2 must share bf16 or fp32")
     _require(w1.is_contiguous() and w1.shape == (E, (2 if gated else 1) * inter, H) and w2.is_contiguous() and w2.shape == (E, H, inter),
              "w1 must be contiguous [E, 2I or I, H] and w2 [E, H, I]")
-    _require(router_weight.dtype == torch.float32 and router_weight.is_contiguous() and router_weight.shape == (E, H),
-             "router_weight must be contiguous fp32 [E, H]")
+    _require(router_weight.dtype == torch.float32 and router_weight.is_contiguous() and router_weight.shape == (rows, H),
+             "router_weight must be contiguous fp32 [router outputs (+ extra rows), H]")
     _f32vec(router_bias, E, "router_bias")
     dev = x.device
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    identity_weight = gate = None
+    if choice is not None:
+        _dev(x, choice.correction)
+        _f32vec(choice.correction, outputs, "correction")
+        _require(choice.groups >= 1 and outputs % choice.groups == 0 and 1 <= choice.keep <= choice.groups, "the outputs must split into equal groups")
+        _require(choice.keep == choice.groups or choice.keep * (outputs // choice.groups) >= top_k, "the kept groups hold fewer outputs than top_k")
+        _require(choice.extra_rows in (0, 1) and 0 <= choice.identity and top_k <= outputs, "extra_rows is 0 or 1")
+        identity_weight = torch.empty(T, dtype=torch.float32, device=dev) if choice.identity else None
+        gate = torch.empty(T, dtype=torch.float32, device=dev) if choice.extra_rows else None
     if T == 0:
-        return out
+        return out if choice is None else (out, identity_weight, gate)
     P = T * top_k
     ids = torch.empty(T, top_k, dtype=torch.int32, device=dev)
     wts = torch.empty(T, top_k, dtype=torch.float32, device=dev)
@@ -1969,9 +2006,15 @@ def moe_routed_forward(x: torch.Tensor, router_weight: torch.Tensor, router_bias
     r = _C.MoeRouteSigmoidArgs()
     r.x, r.router_weight, r.topk_ids, r.topk_weights = _p(x), _p(router_weight), _p(ids), _p(wts)
     r.expert_offsets, r.sorted_pair, r.pair_pos = _p(offsets), _p(sorted_pair), _p(pair_pos)
-    r.num_tokens, r.num_experts, r.top_k, r.hidden, r.act_dtype, r.scale, r.x_stride_t = T, E, top_k, H, _act(x), route_scale, x.stride(0)
+    r.num_tokens, r.num_experts, r.top_k, r.hidden, r.act_dtype, r.scale, r.x_stride_t = T, outputs, top_k, H, _act(x), route_scale, x.stride(0)
     r.router_bias, r.score_mode = _p(router_bias), score_mode
+    if choice is not None:
+        r.num_groups, r.keep_groups, r.first_identity, r.extra_rows = choice.groups, choice.keep, (E if choice.identity else 0), choice.extra_rows
+        r.correction, r.identity_weight, r.extra_out = _p(choice.correction), _p(identity_weight), _p(gate)
     _C.check(lib.hymeta_moe_route_sigmoid(C.byref(r), st), "hymeta_moe_route_sigmoid")
+
+    def result(o):
+        return o if choice is None else (o, identity_weight, gate)
 
     if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and n1 % 64 == 0 and E <= 64 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
         h1 = torch.empty(P, n1, dtype=torch.bfloat16, device=dev)
@@ -1981,7 +2024,7 @@ def moe_routed_forward(x: torch.Tensor, router_weight: torch.Tensor, router_bias
         g.local_expert_begin, g.local_expert_end = 0, E
         g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), h1.stride(0), w1.stride(0)
         _C.check(lib.hymeta_moe_gemm(C.byref(g), st), "hymeta_moe_gemm (w1)")
-        hact = clamped_glu(h1, limit, alpha) if gated else relu_squared(h1, out=h1)
+        hact = clamped_glu(h1, limit, alpha) if expert_act == "clamped_glu" else silu_mul(h1) if gated else relu_squared(h1, out=h1)
         y = torch.empty(P, H, dtype=torch.bfloat16, device=dev)
         d = _C.MoeGemmArgs()
         d.x, d.x_stride_m, d.weights, d.out, d.expert_offsets = _p(hact), hact.stride(0), _p(w2), _p(y), _p(offsets)
@@ -1995,14 +2038,14 @@ def moe_routed_forward(x: torch.Tensor, router_weight: torch.Tensor, router_bias
         c.num_tokens, c.hidden, c.top_k = T, H, top_k
         c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
         _C.check(lib.hymeta_moe_combine(C.byref(c), st), "hymeta_moe_combine")
-        return out
+        return result(out)
 
     act = _DT[x.dtype]
     hact = torch.empty(P, inter, dtype=x.dtype, device=dev)
     g = _C.MoeGemmAnyArgs()
     g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w1), _p(hact), _p(offsets)
     g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N, g.num_experts, g.act_dtype = _p(sorted_pair), top_k, P, H, inter, E, act
-    g.gated = _C.GLU_CLAMPED if gated else _C.GLU_RELU2
+    g.gated = _C.GLU_CLAMPED if expert_act == "clamped_glu" else _C.GLU_SILU if gated else _C.GLU_RELU2
     g.act_limit, g.act_alpha = limit, alpha
     g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), hact.stride(0), w1.stride(0)
     _C.check(lib.hymeta_moe_gemm_any(C.byref(g), st), "hymeta_moe_gemm_any (w1)")
@@ -2018,7 +2061,7 @@ def moe_routed_forward(x: torch.Tensor, router_weight: torch.Tensor, router_bias
     c.num_tokens, c.width, c.top_k, c.act_dtype = T, H, top_k, act
     c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
     _C.check(lib.hymeta_moe_combine_any(C.byref(c), st), "hymeta_moe_combine_any")
-    return out
+    return result(out)
 
 
 def silu_mul(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -2141,3 +2184,153 @@ def talk_qkv_prep(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         a.positions = _p(positions)
     _C.check(_C.load().hymeta_talk_qkv_prep(C.byref(a), _stream(qkv)), "hymeta_talk_qkv_prep")
     return q_out
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of parallel-layer designs (one norm, mixer and feed-forward side by side) with rotate-half rotary
+# attention, retention and state-space mixers.
+# ---------------------------------------------------------------------------
+def stream_add_norm_(x: torch.Tensor, terms: Sequence[Tuple[torch.Tensor, float, Optional[torch.Tensor]]], norm_scale: Optional[float],
+                     eps: float, out_dtype: Optional[torch.dtype] = None, norm_weight: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``x += sum_i coef_i * (row_scale_i[t] or 1) * y_i`` on the fp32 rows ``x [T, W]``, in place; ``terms`` lists ``(y_i [T, W]
+    activations, coef_i, row_scale_i fp32 [T] or None)``.  With ``norm_scale`` also returns ``x / sqrt(mean(x^2) + eps) *
+    norm_scale (* norm_weight)`` of the new rows in ``out_dtype``: a parallel layer's sum and the next norm, one launch."""
+    _require(x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1, "x must be row-contiguous fp32 [T, W]")
+    _require(len(terms) <= _C.STREAM_MAX_TERMS, f"at most {_C.STREAM_MAX_TERMS} terms")
+    _require(terms or norm_scale is not None, "nothing to do")
+    T, W = x.shape
+    act = out_dtype
+    a = _C.StreamAddNormArgs()
+    for i, (y, coef, row_scale) in enumerate(terms):
+        _dev(x, y, row_scale)
+        _require(y.shape == (T, W) and y.stride(1) == 1 and y.dtype in _DT and (act is None or act == y.dtype), "terms must be row-contiguous [T, W] of one type")
+        _f32vec(row_scale, T, "row_scale")
+        act = y.dtype
+        a.y[i], a.row_scale[i], a.coef[i], a.y_stride_t[i] = _p(y), _p(row_scale), float(coef), y.stride(0)
+    _require(act in _DT, "out_dtype must be bf16 or fp32")
+    _f32vec(norm_weight, W, "norm_weight")
+    h = torch.empty(T, W, dtype=act, device=x.device) if norm_scale is not None else None
+    a.x, a.norm_weight, a.h_out = _p(x), _p(norm_weight), _p(h)
+    a.num_tokens, a.width, a.num_terms, a.act_dtype = T, W, len(terms), _DT[act]
+    a.eps, a.norm_scale, a.x_stride_t = eps, float(norm_scale or 0.0), x.stride(0)
+    _C.check(_C.load().hymeta_stream_add_norm(C.byref(a), _stream(x)), "hymeta_stream_add_norm")
+    return h
+
+
+def rotary_cache_(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int, rot_dims: int,
+                  rot_freqs: Optional[torch.Tensor], k_scale: float = 1.0, kv_cache: Optional[torch.Tensor] = None,
+                  slot_mapping: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+                  query_start_loc: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None) -> None:
+    """On the rows ``qkv [T, H D + G D + G Dv (+ ...)]`` of a fused projection, in place: dimensions ``i`` and ``i + rot_dims / 2``
+    of every query and key head turn by ``position * rot_freqs[i]`` (``rot_freqs`` float64 ``[rot_dims / 2]``), keys are
+    multiplied by ``k_scale``, and with ``kv_cache [blocks, block_size, G, D + Dv]`` the keys and values are written at
+    ``slot_mapping``.  Positions: ``positions`` (int64) or the rows' places in their sequences (``query_start_loc``, ``seq_lens``)."""
+    _dev(qkv, rot_freqs, kv_cache, slot_mapping, positions, query_start_loc, seq_lens)
+    H, G, D, Dv = num_heads, num_kv_heads, head_dim, v_dim
+    T = qkv.shape[0]
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= (H + G) * D + (G * Dv if kv_cache is not None else 0),
+             "qkv must be row-contiguous [T, H D + G D + G Dv (+ ...)]")
+    _require(rot_dims % 2 == 0 and 0 <= rot_dims <= D, "rot_dims must be even and fit a head")
+    a = _C.RotaryCacheArgs()
+    if rot_dims:
+        _require(rot_freqs is not None and rot_freqs.dtype == torch.float64 and rot_freqs.is_contiguous() and rot_freqs.numel() == rot_dims // 2,
+                 "rot_freqs must be contiguous float64 [rot_dims / 2]")
+        if positions is not None:
+            _require(positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T, "positions must be int64 [T]")
+        else:
+            _require(query_start_loc is not None and seq_lens is not None, "positions or the step's sequence layout")
+    if positions is None and query_start_loc is not None:
+        S = query_start_loc.numel() - 1
+        _i32vec(query_start_loc, S + 1, "query_start_loc")
+        _i32vec(seq_lens, S, "seq_lens")
+        a.query_start_loc, a.seq_lens, a.num_seqs = _p(query_start_loc), _p(seq_lens), S
+    a.qkv, a.rot_freqs, a.positions = _p(qkv), _p(rot_freqs), _p(positions)
+    a.num_tokens, a.num_heads, a.num_kv_heads, a.head_dim, a.v_dim, a.rot_dims = T, H, G, D, Dv, rot_dims
+    a.act_dtype, a.k_scale, a.qkv_stride_t, a.block_size = _act(qkv), float(k_scale), qkv.stride(0), 1
+    if kv_cache is not None:
+        _require(kv_cache.dtype == qkv.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4 and kv_cache.shape[2:] == (G, D + Dv),
+                 "kv_cache must be contiguous [blocks, block_size, G, D + Dv]")
+        _require(slot_mapping is not None and slot_mapping.dtype == torch.int64 and slot_mapping.is_contiguous() and slot_mapping.numel() == T,
+                 "slot_mapping must be int64 [T]")
+        a.kv_cache, a.slot_mapping, a.num_blocks, a.block_size = _p(kv_cache), _p(slot_mapping), kv_cache.shape[0], kv_cache.shape[1]
+    _C.check(_C.load().hymeta_rotary_cache(C.byref(a), _stream(qkv)), "hymeta_rotary_cache")
+
+
+def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], conv_state: Optional[torch.Tensor],
+                     query_start_loc: torch.Tensor, context_lens: torch.Tensor, slot_idx: Optional[torch.Tensor],
+                     dt_in: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None, a_log: Optional[torch.Tensor] = None):
+    """``silu(bias + sum_j weight[:, j] x[t - taps + 1 + j])`` per channel over each sequence's rows of ``x [T, C]`` (a view
+    with any row stride); ``weight`` fp32 ``[C, taps]``; ``conv_state [slots, taps - 1, C]`` (x's type) carries a sequence's
+    last input rows between steps, in place.  With ``dt_in [T, heads]`` also returns fp32 ``softplus(dt_in + dt_bias)`` and
+    ``-exp(a_log) dt log2(e)``, both ``[T, heads]``: a state-space layer's step sizes and log2 decays.  Returns ``out`` or
+    ``(out, dt, log2_decay)``."""
+    _dev(x, weight, bias, conv_state, query_start_loc, context_lens, slot_idx, dt_in, dt_bias, a_log)
+    _require(x.dim() == 2 and x.stride(1) == 1 and x.dtype in _DT, "x must be row-contiguous [T, C], bf16 or fp32")
+    T, Cn = x.shape
+    taps = weight.shape[1]
+    _require(weight.dtype == torch.float32 and weight.is_contiguous() and weight.shape == (Cn, taps) and 1 <= taps <= _C.CONV_MAX_TAPS,
+             f"weight must be contiguous fp32 [C, taps <= {_C.CONV_MAX_TAPS}]")
+    _f32vec(bias, Cn, "bias")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(context_lens, S, "context_lens")
+    out = torch.empty(T, Cn, dtype=x.dtype, device=x.device)
+    a = _C.CausalConvArgs()
+    a.x, a.weight, a.bias, a.out = _p(x), _p(weight), _p(bias), _p(out)
+    a.query_start_loc, a.context_lens = _p(query_start_loc), _p(context_lens)
+    a.num_tokens, a.num_seqs, a.channels, a.taps, a.act_dtype, a.x_stride_t = T, S, Cn, taps, _act(x), x.stride(0)
+    if conv_state is not None and taps > 1:
+        _require(slot_idx is not None, "conv_state needs slot_idx")
+        _i32vec(slot_idx, S, "slot_idx")
+        _require(conv_state.dtype == x.dtype and conv_state.is_contiguous() and conv_state.dim() == 3 and conv_state.shape[1:] == (taps - 1, Cn),
+                 "conv_state must be contiguous [slots, taps - 1, C] of x's type")
+        a.conv_state, a.slot_idx = _p(conv_state), _p(slot_idx)
+    dt = ld = None
+    if dt_in is not None:
+        Hh = dt_in.shape[1]
+        _require(dt_in.dim() == 2 and dt_in.shape[0] == T and dt_in.stride(1) == 1 and dt_in.dtype == x.dtype, "dt_in must be [T, heads] of x's type")
+        _f32vec(dt_bias, Hh, "dt_bias")
+        _f32vec(a_log, Hh, "a_log")
+        _require(dt_bias is not None and a_log is not None, "dt_in comes with dt_bias and a_log")
+        dt = torch.empty(T, Hh, dtype=torch.float32, device=x.device)
+        ld = torch.empty(T, Hh, dtype=torch.float32, device=x.device)
+        a.dt_in, a.dt_bias, a.a_log, a.dt_out, a.log2_decay_out, a.dt_heads, a.dt_stride_t = _p(dt_in), _p(dt_bias), _p(a_log), _p(dt), _p(ld), Hh, dt_in.stride(0)
+    _C.check(_C.load().hymeta_causal_conv(C.byref(a), _stream(x)), "hymeta_causal_conv")
+    return out if dt_in is None else (out, dt, ld)
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, query_start_loc: torch.Tensor,
+               context_lens: torch.Tensor, slot_idx: torch.Tensor, max_query_len: int, decay: Optional[torch.Tensor] = None,
+               log2_decay: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None, skip: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``S_t = a_t S_{t-1} + b_t k_t v_t^T``, ``out_t = S_t^T q_t + skip[h] v_t`` over a step's rows: ``q, k [T, Hqk, D]`` and
+    ``v [T, H, Dv]`` (views with any row stride; head ``h`` reads query / key head ``h // (H / Hqk)``), ``state`` fp32
+    ``[slots, H, D, Dv]`` read where ``context_lens > 0`` and written.  ``a_t``: ``decay [H]`` for every token, or
+    ``2 ** log2_decay[t, h]``; ``b_t``: ``v_scale [T, H]`` or 1.  Returns fp32 ``[T, H Dv]``."""
+    _dev(q, k, v, state, query_start_loc, context_lens, slot_idx, decay, log2_decay, v_scale, skip)
+    _require(q.dim() == 3 and k.shape == q.shape and v.dim() == 3 and q.dtype == k.dtype == v.dtype and q.dtype in _DT, "q, k [T, Hqk, D] and v [T, H, Dv] of one type")
+    T, Hqk, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    for t_, n_ in ((q, D), (k, D), (v, Dv)):
+        _require(t_.shape[0] == T and t_.stride(2) == 1 and t_.stride(1) == n_, "heads must be contiguous in a row")
+    _require(H % Hqk == 0, "the heads must split over the query / key heads")
+    _require(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 4 and state.shape[1:] == (H, D, Dv),
+             "state must be contiguous fp32 [slots, H, D, Dv]")
+    _require((decay is None) != (log2_decay is None), "decay [H] or log2_decay [T, H]")
+    _f32vec(decay, H, "decay")
+    _f32vec(log2_decay, T * H, "log2_decay")
+    _f32vec(v_scale, T * H, "v_scale")
+    _f32vec(skip, H, "skip")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(context_lens, S, "context_lens")
+    _i32vec(slot_idx, S, "slot_idx")
+    out = torch.empty(T, H * Dv, dtype=torch.float32, device=q.device)
+    a = _C.DecayScanArgs()
+    a.q, a.k, a.v, a.state, a.out = _p(q), _p(k), _p(v), _p(state), _p(out)
+    a.decay, a.log2_decay, a.v_scale, a.skip = _p(decay), _p(log2_decay), _p(v_scale), _p(skip)
+    a.query_start_loc, a.context_lens, a.slot_idx = _p(query_start_loc), _p(context_lens), _p(slot_idx)
+    a.num_tokens, a.num_seqs, a.num_heads, a.num_qk_heads, a.head_dim, a.v_dim = T, S, H, Hqk, D, Dv
+    a.act_dtype, a.max_query_len = _act(q), max_query_len
+    a.q_stride_t, a.k_stride_t, a.v_stride_t = q.stride(0), k.stride(0), v.stride(0)
+    _C.check(_C.load().hymeta_decay_scan(C.byref(a), _stream(q)), "hymeta_decay_scan")
+    return out

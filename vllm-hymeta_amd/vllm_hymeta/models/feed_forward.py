@@ -8,6 +8,9 @@
 ``SiluGluMLP``      ``W_down (silu(W_gate h + b_gate) (W_up h + b_up)) + b_down``, bf16 or fp32
 ``Relu2RoutedMoE``  experts ``W_down max(W_up h, 0)^2`` chosen by the largest router logits ``W_r h + b_r``, weighing the
                     softmax over the chosen logits alone
+``GroupedSoftmaxMoE``  silu-gated experts weighed by the softmax over ALL router outputs (not renormalised), chosen by
+                    corrected scores within the best groups of outputs; the last outputs are identity experts; a shared
+                    expert behind a sigmoid gate of one number per token
 
 Beside ``HymetaMoE`` (``moe.py``: softmax router, silu experts) and ``TableMoE`` (``table_moe.py``: no router network);
 the expert stacks ``w13 [E, 2I, H]`` / ``w2 [E, H, I]`` are theirs.
@@ -88,3 +91,35 @@ class Relu2RoutedMoE(torch.nn.Module):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return hip_ops.moe_routed_forward(h, self.router_weight, self.router_bias, self.w1, self.w2, self.top_k,
                                           hip_ops.ROUTE_SOFTMAX_CHOSEN, 1.0, "relu2")
+
+
+class GroupedSoftmaxMoE(torch.nn.Module):
+    """``s = softmax(W_r h)`` over ``experts + identity`` outputs; the ``top_k`` largest ``s + correction`` among the outputs
+    of the ``keep`` groups (of ``groups`` equal runs of neighbours) whose best corrected score is largest are chosen; the
+    output is ``sum_chosen s_e expert_e(h)`` with ``expert_e(h) = W_down (silu(W_gate h) W_up h)``, or ``h`` itself for the
+    last ``identity`` outputs, plus ``sigmoid(w_sg . h) shared(h)``."""
+
+    def __init__(self, router_weight: torch.Tensor, correction: Optional[torch.Tensor], w13: torch.Tensor, w2: torch.Tensor, top_k: int,
+                 groups: int, keep: int, identity: int, shared: Optional[SiluGluMLP] = None, shared_gate: Optional[torch.Tensor] = None):
+        """``router_weight [experts + identity, H]``, ``shared_gate [1, H]`` (with ``shared``)."""
+        super().__init__()
+        if (shared is None) != (shared_gate is None):
+            raise ValueError("the shared expert comes with its gate")
+        rows = router_weight.float() if shared_gate is None else torch.cat([router_weight.float(), shared_gate.float().reshape(1, -1)], 0)
+        self.register_buffer("router_rows", rows.contiguous())           # the router runs in fp32; the gate's row rides behind it
+        self.register_buffer("correction", None if correction is None else correction.float().contiguous())
+        self.register_buffer("w13", w13.contiguous())
+        self.register_buffer("w2", w2.contiguous())
+        self.top_k, self.groups, self.keep, self.identity, self.shared = int(top_k), int(groups), int(keep), int(identity), shared
+
+    def forward(self, h: torch.Tensor):
+        """Terms for whoever adds them to the stream: the routed sum, ``identity_weight[t] h[t]``, the gated shared expert."""
+        choice = hip_ops.GroupedChoice(self.correction, self.groups, self.keep, self.identity, 0 if self.shared is None else 1)
+        y, identity_weight, gate = hip_ops.moe_routed_forward(h, self.router_rows, None, self.w13, self.w2, self.top_k,
+                                                              hip_ops.ROUTE_SOFTMAX_GROUPED, 1.0, "silu_glu", choice=choice)
+        terms = [(y, 1.0, None)]
+        if identity_weight is not None:
+            terms.append((h, 1.0, identity_weight))
+        if self.shared is not None:
+            terms.append((self.shared(h), 1.0, gate))
+        return terms

@@ -31,6 +31,11 @@ def _lidizen_config(model_dir: str):
     return LidizenConfig.from_pretrained(model_dir)
 
 
+def _dapuzen_config(model_dir: str):
+    from .models.configuration_dapuzen import DapuzenConfig
+    return DapuzenConfig.from_pretrained(model_dir)
+
+
 def _gla_swa_config(model_dir: str):
     from .model_for_7B.configuration_gla_swa import GLAswaConfig
     with open(os.path.join(model_dir, "config.json")) as f:
@@ -45,6 +50,8 @@ register("Geponex", "vllm_hymeta.models.modeling_geponex:GeponexForCausalLM", _g
 register("GeponexForCausalLM", "vllm_hymeta.models.modeling_geponex:GeponexForCausalLM", _geponex_config)
 register("Lidizen", "vllm_hymeta.models.modeling_lidizen:LidizenForCausalLM", _lidizen_config)
 register("LidizenForCausalLM", "vllm_hymeta.models.modeling_lidizen:LidizenForCausalLM", _lidizen_config)
+register("Dapuzen", "vllm_hymeta.models.modeling_dapuzen:DapuzenForCausalLM", _dapuzen_config)
+register("DapuzenForCausalLM", "vllm_hymeta.models.modeling_dapuzen:DapuzenForCausalLM", _dapuzen_config)
 register("GLAswaForCausalLM", "vllm_hymeta.model_for_7B.modeling_gla_swa:GLAswaForCausalLM", _gla_swa_config)
 
 
@@ -78,6 +85,8 @@ _KERNEL_SOURCES = {
                            "moe_table", "moe", "glue", "dense_gemm", "stream_gemm", "tall_gemm"),
     "LidizenForCausalLM": ("api_misc", "hyper_stream", "talk_attn", "sink_attn", "gated_ops", "moe_sigmoid", "moe_table", "moe", "glue",
                            "dense_gemm", "stream_gemm", "tall_gemm"),
+    "DapuzenForCausalLM": ("api_misc", "norm_conv", "parallel_ops", "decay_scan", "lightning", "sink_attn", "gated_ops", "moe_sigmoid",
+                           "moe_table", "moe", "glue", "dense_gemm", "stream_gemm", "tall_gemm"),
 }
 
 
