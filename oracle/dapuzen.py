@@ -296,7 +296,7 @@ def dapuzen_random_weights(cfg: dict, seed: int = 0, std: float = 1.0) -> Dict[s
     W = cfg["width"]
 
     def rnd(*shape, s=1.0):
-        return (torch.randn(*shape, generator=g) * s * std).to(torch.bfloat16).float()
+        return (torch.randn(shape, generator=g) * s * std).to(torch.bfloat16).float()
 
     def lin(o, i):
         return rnd(o, i, s=i ** -0.5)
