@@ -131,6 +131,230 @@ __global__ __launch_bounds__(256) void decay_scan_step_kernel(hymeta_decay_scan_
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// bf16 portions in chunks of 64 rows on the matrix cores.  With S the state before the chunk, i and j rows of the
+// chunk, n its number of rows, l_j the log2 decays and c_i = l_0 + ... + l_i their running sums:
+//   o_i   = 2^(c_i) S^T q_i + sum_{j <= i} 2^(c_i - c_j) b_j (q_i . k_j) v_j + skip v_i
+//   S_new = 2^(c_{n-1}) S + sum_j 2^(c_{n-1} - c_j) b_j k_j v_j^T
+// grid = (heads, sequences, value columns in slices of 32); 4 waves, each with 16 rows of the chunk.  The state
+// slice stays fp32 in registers, transposed (S^T [c][d]: a lane holds 4 value columns of one d), 16 x 16 blocks dealt
+// over the waves; what enters a matrix product from fp32 (the decayed weights, the decayed keys, the state) goes in as
+// hi + lo bf16 parts, two products, so that it keeps 16 bits of mantissa.  Every wave keeps the chunk's running sums in
+// its lanes (lane = row of the chunk), so the decays cost shuffles and no LDS.
+// ------------------------------------------------------------------------------------------------
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+constexpr int kChunk = HYMETA_SCAN_CHUNK, kSliceV = 32;
+constexpr int kChunkMinRows = 8;            // shorter portions go token by token
+constexpr float kMinLog2 = -1.0e4f;         // a decay of 0 (or an overflowed step size): finite, so that differences of sums stay numbers
+
+__device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+
+template <int D>
+__global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan_args a, int min_rows) {
+  constexpr int PK = D + 8, PT = kChunk + 8, NBW = (2 * D / 16) / 4;
+  __shared__ __attribute__((aligned(16))) uint16_t sk[kChunk * PK];          // k, a row per key
+  __shared__ __attribute__((aligned(16))) uint16_t skt[2][D * PT];           // decayed keys, transposed [d][key], hi / lo
+  __shared__ __attribute__((aligned(16))) uint16_t svt[kSliceV * PT];        // v of the slice, transposed [c][key]
+  __shared__ __attribute__((aligned(16))) uint16_t sst[2][kSliceV * PK];     // state^T [c][d], hi / lo
+  const int h = blockIdx.x, s = blockIdx.y, vs = blockIdx.z;
+  const int r0 = a.query_start_loc[s], rows = a.query_start_loc[s + 1] - r0;
+  if (rows < min_rows) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g4 = lane >> 4;
+  const int H = a.num_heads, Dv = a.v_dim;
+  const int g = h / (H / a.num_qk_heads);
+  const int slot = a.slot_idx[s];
+  float* st = slot >= 0 ? a.state + ((static_cast<int64_t>(slot) * H + h) * D) * Dv + vs * kSliceV : nullptr;
+  const float l2_const = a.decay ? fmaxf(a.decay[h] > 0.f ? log2f(a.decay[h]) : -INFINITY, kMinLog2) : 0.f;
+  const float skip = a.skip ? a.skip[h] : 0.f;
+  const bool carry = st != nullptr && a.context_lens[s] > 0;
+  f32x4v S[NBW];
+#pragma unroll
+  for (int ib = 0; ib < NBW; ++ib) {
+    const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+    S[ib] = carry ? *reinterpret_cast<const f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) : f32x4v{0.f, 0.f, 0.f, 0.f};
+  }
+  auto state_to_lds = [&]() {
+#pragma unroll
+    for (int ib = 0; ib < NBW; ++ib) {
+      const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = S[ib][r];
+        const uint16_t hi = f2bf(v);
+        const int at = (16 * cb + 4 * g4 + r) * PK + 16 * db + n;
+        sst[0][at] = hi;
+        sst[1][at] = f2bf(v - bf2f(hi));
+      }
+    }
+  };
+  state_to_lds();
+  const uint16_t* qp = static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(g) * D;
+  const uint16_t* kp = static_cast<const uint16_t*>(a.k) + static_cast<int64_t>(g) * D;
+  const uint16_t* vp = static_cast<const uint16_t*>(a.v) + static_cast<int64_t>(h) * Dv + vs * kSliceV;
+  // the rows of a chunk as they come from memory: this thread's share of the keys (KPT groups of 8 columns of one row) and
+  // of the value slice, this lane's query fragment, and row `lane`'s log2 decay and input weight; loaded a chunk ahead
+  constexpr int KPT = kChunk * (D / 8) / 256;
+  u32x4 rk[KPT], rv, rq[D / 32];
+  float rl, rb;
+  auto fetch = [&](int c0) {
+    const int nrow = min(kChunk, rows - c0);
+    const int64_t t0 = r0 + c0;
+#pragma unroll
+    for (int u = 0; u < KPT; ++u) {
+      const int idx = tid + 256 * u, j = idx % kChunk, ch = idx / kChunk;
+      rk[u] = u32x4{0u, 0u, 0u, 0u};
+      if (j < nrow) rk[u] = ld16g(kp + (t0 + j) * a.k_stride_t + 8 * ch);
+    }
+    {
+      const int j = tid % kChunk, ch = tid / kChunk;
+      rv = u32x4{0u, 0u, 0u, 0u};
+      if (j < nrow) rv = ld16g(vp + (t0 + j) * a.v_stride_t + 8 * ch);
+    }
+    const int i = 16 * wave + n;
+#pragma unroll
+    for (int sd = 0; sd < D / 32; ++sd) {
+      rq[sd] = u32x4{0u, 0u, 0u, 0u};
+      if (i < nrow) rq[sd] = ld16g(qp + (t0 + i) * a.q_stride_t + 32 * sd + 8 * g4);
+    }
+    rl = 0.f, rb = 0.f;
+    if (lane < nrow) {
+      rl = a.log2_decay ? fmaxf(a.log2_decay[(t0 + lane) * H + h], kMinLog2) : l2_const;
+      rb = a.v_scale ? a.v_scale[(t0 + lane) * H + h] : 1.f;
+    }
+  };
+  static_assert(kChunk * (kSliceV / 8) == 256, "one group of the value slice per thread");
+  fetch(0);
+  for (int c0 = 0; c0 < rows; c0 += kChunk) {
+    const int nrow = min(kChunk, rows - c0);
+    // running sums of the chunk's log2 decays over the wave's lanes (rows past the portion add 0)
+    float cum = rl;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float up = __shfl_up(cum, o, 64);
+      if (lane >= o) cum += up;
+    }
+    const float total = __shfl(cum, nrow - 1, 64);
+    const float bw = rb;
+    // a wave's lanes hold 64 different rows of one 8-column group (row = lane): the transposed 2-byte stores of a wave fall
+    // on consecutive addresses, the row-major 16-byte stores on different banks
+    const float kd = lane < nrow ? __builtin_amdgcn_exp2f(total - cum) * bw : 0.f;
+#pragma unroll
+    for (int u = 0; u < KPT; ++u) {
+      const int idx = tid + 256 * u, j = idx % kChunk, ch = idx / kChunk;
+      st16(&sk[j * PK + 8 * ch], rk[u]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t w = rk[u][e >> 1];
+        const float x = (e & 1 ? hi_bf(w) : lo_bf(w)) * kd;
+        const uint16_t hi = f2bf(x);
+        skt[0][(8 * ch + e) * PT + j] = hi;
+        skt[1][(8 * ch + e) * PT + j] = f2bf(x - bf2f(hi));
+      }
+    }
+    {
+      const int j = tid % kChunk, ch = tid / kChunk;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) svt[(8 * ch + e) * PT + j] = static_cast<uint16_t>(e & 1 ? rv[e >> 1] >> 16 : rv[e >> 1] & 0xffffu);
+    }
+    const int i = 16 * wave + n;                       // this lane's row of the chunk (as a column of the products)
+    bf16x8 q[D / 32];
+#pragma unroll
+    for (int sd = 0; sd < D / 32; ++sd) q[sd] = __builtin_bit_cast(bf16x8, rq[sd]);
+    __syncthreads();
+    if (c0 + kChunk < rows) fetch(c0 + kChunk);        // in flight while this chunk is multiplied
+    {
+      // weights of the chunk's own rows: (q_i . k_j) 2^(c_i - c_j) b_j for j <= i, as hi + lo parts
+      const float cum_i = __shfl(cum, i, 64);
+      uint32_t phi[4][2], plo[4][2];
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        f32x4v sc = f32x4v{0.f, 0.f, 0.f, 0.f};
+        if (ks <= wave) {
+#pragma unroll
+          for (int sd = 0; sd < D / 32; ++sd)
+            sc = mfma16(__builtin_bit_cast(bf16x8, ld16(&sk[(16 * ks + n) * PK + 32 * sd + 8 * g4])), q[sd], sc);
+        }
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int j = 16 * ks + 4 * g4 + r;
+          const float cum_j = __shfl(cum, j, 64), b_j = __shfl(bw, j, 64);
+          p[r] = (ks <= wave && j <= i) ? sc[r] * __builtin_amdgcn_exp2f(cum_i - cum_j) * b_j : 0.f;
+        }
+#pragma unroll
+        for (int r2 = 0; r2 < 2; ++r2) {
+          const uint32_t hi = pack_bf16x2(p[2 * r2], p[2 * r2 + 1]);
+          phi[ks][r2] = hi;
+          plo[ks][r2] = pack_bf16x2(p[2 * r2] - lo_bf(hi), p[2 * r2 + 1] - hi_bf(hi));
+        }
+      }
+      f32x4v o[2];
+      const float row_decay = __builtin_amdgcn_exp2f(cum_i);
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        // the state before the chunk
+        f32x4v x = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sd = 0; sd < D / 32; ++sd) {
+          x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[0][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
+          x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[1][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
+        }
+        f32x4v acc = x * row_decay;
+        if (skip != 0.f) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] = fmaf(skip, bf2f(svt[(16 * cb + 4 * g4 + r) * PT + i]), acc[r]);
+        }
+#pragma unroll
+        for (int kp2 = 0; kp2 < 2; ++kp2) {
+          if (2 * kp2 > wave) continue;
+          // k index 8 g4 + e of the product: keys 32 kp2 + 4 g4 + e for e < 4, 32 kp2 + 16 + 4 g4 + e - 4 after
+          const u32x2 v0 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp2 + 4 * g4]);
+          const u32x2 v1 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp2 + 16 + 4 * g4]);
+          const bf16x8 vf = __builtin_bit_cast(bf16x8, (u32x4{v0[0], v0[1], v1[0], v1[1]}));
+          acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{phi[2 * kp2][0], phi[2 * kp2][1], phi[2 * kp2 + 1][0], phi[2 * kp2 + 1][1]})), acc);
+          acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{plo[2 * kp2][0], plo[2 * kp2][1], plo[2 * kp2 + 1][0], plo[2 * kp2 + 1][1]})), acc);
+        }
+        o[cb] = acc;
+      }
+      if (i < nrow) {
+        float* orow = a.out + static_cast<int64_t>(r0 + c0 + i) * H * Dv + static_cast<int64_t>(h) * Dv + vs * kSliceV;
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) *reinterpret_cast<f32x4v*>(orow + 16 * cb + 4 * g4) = o[cb];
+      }
+    }
+    // the state after the chunk
+    const float chunk_decay = __builtin_amdgcn_exp2f(total);
+#pragma unroll
+    for (int ib = 0; ib < NBW; ++ib) {
+      const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+      f32x4v acc = S[ib] * chunk_decay;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, ld16(&svt[(16 * cb + n) * PT + 32 * kk + 8 * g4]));
+        acc = mfma16(vf, __builtin_bit_cast(bf16x8, ld16(&skt[0][(16 * db + n) * PT + 32 * kk + 8 * g4])), acc);
+        acc = mfma16(vf, __builtin_bit_cast(bf16x8, ld16(&skt[1][(16 * db + n) * PT + 32 * kk + 8 * g4])), acc);
+      }
+      S[ib] = acc;
+    }
+    __syncthreads();            // every wave is done with this chunk's tiles and with the old state's image
+    state_to_lds();             // (made visible by the barrier after the next chunk's staging)
+  }
+  if (st != nullptr) {
+#pragma unroll
+    for (int ib = 0; ib < NBW; ++ib) {
+      const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+      *reinterpret_cast<f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) = S[ib];
+    }
+  }
+}
+
+inline bool chunk_shape(const hymeta_decay_scan_args& a) {
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  return a.act_dtype == HYMETA_BF16 && (a.head_dim == 32 || a.head_dim == 64 || a.head_dim == 128) && a.v_dim % kSliceV == 0 &&
+         a.q_stride_t % 8 == 0 && a.k_stride_t % 8 == 0 && a.v_stride_t % 8 == 0 && aligned(a.q) && aligned(a.k) && aligned(a.v) &&
+         aligned(a.state) && aligned(a.out) && a.v_dim / kSliceV <= 65535;
+}
+
 inline bool step_shape(const hymeta_decay_scan_args& a) {
   const int dv4 = a.v_dim / 4;
   const int bytes = a.act_dtype == HYMETA_BF16 ? 2 : 4;
@@ -168,6 +392,13 @@ extern "C" int hymeta_decay_scan(const hymeta_decay_scan_args* args, hymeta_stre
   if (a.q_stride_t < qk || a.k_stride_t < qk || a.v_stride_t < static_cast<int64_t>(a.num_heads) * a.v_dim) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
   int max_rows = 0x7fffffff;
+  if (chunk_shape(a) && a.max_query_len >= kChunkMinRows) {
+    const dim3 grid(a.num_heads, a.num_seqs, a.v_dim / kSliceV);
+    if (a.head_dim == 32) hipLaunchKernelGGL(decay_scan_chunk_kernel<32>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    else if (a.head_dim == 64) hipLaunchKernelGGL(decay_scan_chunk_kernel<64>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    else hipLaunchKernelGGL(decay_scan_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    max_rows = kChunkMinRows - 1;
+  }
   int min_rows = 1;
   if (step_shape(a)) {
     const dim3 grid(a.num_heads, a.num_seqs);

@@ -1710,7 +1710,7 @@ def moe_table_forward(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Ten
         c.num_tokens, c.hidden, c.top_k = T, H, top
         c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
         _C.check(lib.hymeta_moe_combine(C.byref(c), st), "hymeta_moe_combine")
-        return result(out)
+        return out
 
     act = _DT[x.dtype]
     hact = torch.empty(P, inter, dtype=x.dtype, device=dev)
