@@ -56,11 +56,12 @@ def parse():
     ap.add_argument("--gla-state", choices=("kv_head", "query_head"), default="kv_head",
                     help="GLA state layout: one state per key/value head (the package's default; the 7 query heads "
                          "of a group hold identical states) or one per query head (the reference's cache shape)")
-    ap.add_argument("--design", choices=("hymeta", "sonuzen", "geponex", "lidizen"), default="hymeta",
+    ap.add_argument("--design", choices=("hymeta", "sonuzen", "geponex", "lidizen", "dapuzen"), default="hymeta",
                     help="hymeta: the headline benchmark (default).  sonuzen: the side benchmark of the Sonuzen design beside the 7B "
                          "family at equal layer sizes (bench_sonuzen.py): prefill and decode throughput and a per-kernel roofline table.  "
                          "geponex: the same for the Geponex design beside Sonuzen (bench_geponex.py).  "
-                         "lidizen: the same for the Lidizen design beside Sonuzen (bench_lidizen.py)")
+                         "lidizen: the same for the Lidizen design beside Sonuzen (bench_lidizen.py).  "
+                         "dapuzen: the same for the Dapuzen design beside Geponex (bench_dapuzen.py)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the 32k TTFT / single-request latency side measurements")
     ap.add_argument("--prefill-ctx", type=int, default=32768)
@@ -641,6 +642,9 @@ def main():
     if args.design == "lidizen":
         import bench_lidizen
         return bench_lidizen.main(args)
+    if args.design == "dapuzen":
+        import bench_dapuzen
+        return bench_dapuzen.main(args)
 
     B, total = args.batch, args.warmup + args.steps
     model = build_model_7b(dev, args.quant, max_num_seqs=B, gla_state=args.gla_state)

@@ -243,8 +243,11 @@ def test_one_key_decides_at_the_edges_of_the_window(dtype, D, Dv, page):
 def test_causal_convolution_in_portions_carries_its_inputs(dtype, C, taps, heads):
     from vllm_hymeta import hip_ops
     g = torch.Generator().manual_seed(C + taps)
-    lens = {0: 37, 1: 1, 2: 12}
-    xs = {k: torch.randn(n, C + heads + 5, generator=g).to(dtype) for k, n in lens.items()}      # a wider row: the stride shows
+    lens = {0: 90, 1: 1, 2: 45}
+    row = C + heads + 5                                          # a wider row: the stride shows
+    if C % 4 == 0:
+        row = (row + 3) // 4 * 4                                 # ... in whole fours where the channels are: the strips of rows run
+    xs = {k: torch.randn(n, row, generator=g).to(dtype) for k, n in lens.items()}
     w = torch.randn(C, taps, generator=g) * taps ** -0.5
     b = torch.randn(C, generator=g) * 0.1
     dt_bias, a_log = torch.randn(heads, generator=g), torch.randn(heads, generator=g) * 0.5 - 1
@@ -265,7 +268,8 @@ def test_causal_convolution_in_portions_carries_its_inputs(dtype, C, taps, heads
             r += n
         return out
 
-    got = in_steps(lens, [[(0, 2)], [(0, 1), (1, 1)], [(0, 1), (2, 4)], [(0, 3), (2, 1)], [(2, 7), (0, 30)]], run)
+    # (the last step: a sequence that ends inside a strip of rows, the next one starting there with a state of its own)
+    got = in_steps(lens, [[(0, 2)], [(0, 1), (1, 1)], [(0, 1), (2, 4)], [(0, 3), (2, 1)], [(2, 7), (0, 30)], [(0, 53), (2, 33)]], run)
     tol = 2e-6 if dtype == torch.float32 else 6e-3
     for k in lens:
         assert rel_err(got[k], refs[k]) < tol, k

@@ -103,6 +103,43 @@ __global__ __launch_bounds__(256) void gated_rms_norm_kernel(hymeta_gated_rms_no
   }
 }
 
+// Narrow groups (a head's output): a wave per (row, group), the group's columns in the lanes' registers, no barrier.
+constexpr int kGatedWavePerLane = 16, kGatedWaveCols = 64 * kGatedWavePerLane;
+
+template <typename A>
+__global__ __launch_bounds__(256) void gated_rms_norm_wave_kernel(hymeta_gated_rms_norm_args a, int groups) {
+  typedef typename A::elem elem;
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, grp = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (grp >= groups) return;
+  const int width = a.width / groups, c0 = grp * width;
+  const float* x = a.x + t * a.width + c0;
+  const elem* g = static_cast<const elem*>(a.gate) + t * a.gate_stride_t + c0;
+  const float* weight = a.weight ? a.weight + c0 : nullptr;
+  elem* out = static_cast<elem*>(a.out) + t * a.width + c0;
+  const bool silu = a.gate_act == HYMETA_GATE_SILU, first = a.gate_first != 0;
+  float xv[kGatedWavePerLane], gv[kGatedWavePerLane];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < kGatedWavePerLane; ++u) {
+    const int c = lane + 64 * u;
+    if (64 * u >= width) { xv[u] = 0.f, gv[u] = 0.f; continue; }
+    xv[u] = c < width ? x[c] : 0.f;
+    const float raw = c < width ? A::ld(g + c) : 0.f;
+    const float sg = sigmoid_exact(raw);
+    gv[u] = silu ? raw * sg : sg;
+    if (first) xv[u] *= gv[u], gv[u] = 1.f;
+    ss = fmaf(xv[u], xv[u], ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(width) + a.eps);
+#pragma unroll
+  for (int u = 0; u < kGatedWavePerLane; ++u) {
+    const int c = lane + 64 * u;
+    if (c < width) A::st(out + c, xv[u] * inv * (weight ? weight[c] : 1.f) * gv[u]);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // bf16 portions in chunks of 64 rows on the matrix cores.  With S the state before the chunk, i and j rows of the
 // chunk, n its number of rows and L = decay:
@@ -511,6 +548,12 @@ extern "C" int hymeta_gated_rms_norm(const hymeta_gated_rms_norm_args* args, hym
   if (a.width % groups != 0 || groups > 65535) return HYMETA_ERR_INVALID_ARG;
   if (a.gate_act != HYMETA_GATE_SIGMOID && a.gate_act != HYMETA_GATE_SILU) return HYMETA_ERR_UNSUPPORTED;
   hipStream_t st = begin_launches(stream);
+  if (groups > 1 && a.width / groups <= kGatedWaveCols) {
+    const dim3 grid(a.num_tokens, (groups + 3) / 4);
+    if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(gated_rms_norm_wave_kernel<ActBf16>, grid, dim3(256), 0, st, a, groups);
+    else hipLaunchKernelGGL(gated_rms_norm_wave_kernel<ActF32>, grid, dim3(256), 0, st, a, groups);
+    return launch_status();
+  }
   const bool cached = a.width / groups <= kGatedCached;
   if (a.act_dtype == HYMETA_BF16) {
     if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, true>), dim3(a.num_tokens, groups), dim3(256), 0, st, a);

@@ -9,9 +9,11 @@ namespace hymeta {
 namespace {
 
 // ------------------------------------------------------------------------------------------------ stream add + norm
-constexpr int kAddPerThread = 16;            // rows up to 256 * 16 columns stay in registers between the sum and the norm
+constexpr int kAddVecs = 4;                  // rows up to 256 * 4 * kAddVecs columns stay in registers between the sum and the norm
 
-template <typename A, bool Cached>
+// Vec: a thread takes runs of four consecutive columns (one load per term and run) and keeps them for the norm; otherwise
+// column by column, the stream read again for the norm.
+template <typename A, bool Vec>
 __global__ __launch_bounds__(256) void stream_add_norm_kernel(hymeta_stream_add_norm_args a) {
   typedef typename A::elem elem;
   __shared__ float red[4];
@@ -25,36 +27,53 @@ __global__ __launch_bounds__(256) void stream_add_norm_kernel(hymeta_stream_add_
     scale[i] = on ? a.coef[i] * (a.row_scale[i] ? a.row_scale[i][t] : 1.f) : 0.f;
     y[i] = on ? static_cast<const elem*>(a.y[i]) + t * a.y_stride_t[i] : nullptr;
   }
-  auto summed = [&](int c) {
-    float v = x[c];
-#pragma unroll
-    for (int i = 0; i < HYMETA_STREAM_MAX_TERMS; ++i)
-      if (i < a.num_terms) v = fmaf(scale[i], A::ld(y[i] + c), v);
-    return v;
-  };
   elem* h = a.h_out ? static_cast<elem*>(a.h_out) + t * a.width : nullptr;
   float ss = 0.f;
-  if (Cached) {
-    float v[kAddPerThread];
+  if (Vec) {
+    float v[kAddVecs][4];
 #pragma unroll
-    for (int u = 0; u < kAddPerThread; ++u) {
-      const int c = threadIdx.x + 256 * u;
-      v[u] = c < a.width ? summed(c) : 0.f;
-      if (c < a.width && a.num_terms > 0) x[c] = v[u];
-      ss = fmaf(v[u], v[u], ss);
+    for (int u = 0; u < kAddVecs; ++u) {
+      const int c = 4 * (threadIdx.x + 256 * u);
+      if (c >= a.width) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[u][e] = 0.f;
+        continue;
+      }
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(x + c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[u][e] = xv[e];
+#pragma unroll
+      for (int i = 0; i < HYMETA_STREAM_MAX_TERMS; ++i) {
+        if (i < a.num_terms) {
+          float yv[4];
+          A::ld4(y[i] + c, yv);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[u][e] = fmaf(scale[i], yv[e], v[u][e]);
+        }
+      }
+      if (a.num_terms > 0) *reinterpret_cast<f32x4*>(x + c) = f32x4{v[u][0], v[u][1], v[u][2], v[u][3]};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss = fmaf(v[u][e], v[u][e], ss);
     }
     if (h == nullptr) return;
     ss = block_sum<4>(ss, red);
     const float inv = a.norm_scale / sqrtf(ss / static_cast<float>(a.width) + a.eps);
 #pragma unroll
-    for (int u = 0; u < kAddPerThread; ++u) {
-      const int c = threadIdx.x + 256 * u;
-      if (c < a.width) A::st(h + c, v[u] * inv * (a.norm_weight ? a.norm_weight[c] : 1.f));
+    for (int u = 0; u < kAddVecs; ++u) {
+      const int c = 4 * (threadIdx.x + 256 * u);
+      if (c >= a.width) continue;
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = v[u][e] * inv * (a.norm_weight ? a.norm_weight[c + e] : 1.f);
+      A::st4(h + c, o);
     }
     return;
   }
   for (int c = threadIdx.x; c < a.width; c += 256) {
-    const float v = summed(c);
+    float v = x[c];
+#pragma unroll
+    for (int i = 0; i < HYMETA_STREAM_MAX_TERMS; ++i)
+      if (i < a.num_terms) v = fmaf(scale[i], A::ld(y[i] + c), v);
     if (a.num_terms > 0) x[c] = v;
     ss = fmaf(v, v, ss);
   }
@@ -166,6 +185,93 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(hymeta_causal_conv_arg
   A::st(static_cast<elem*>(a.out) + static_cast<int64_t>(t) * a.channels + c, acc * sigmoid_exact(acc));
 }
 
+// Many rows, channels in whole fours: a thread takes four consecutive channels through a strip of kConvRows rows, the
+// weights and the last taps - 1 inputs in registers (an input row is read once per strip instead of once per tap); a strip
+// may run over the end of a sequence into the next one, whose history it then fetches anew.
+constexpr int kConvRows = 8;
+
+template <typename A>
+__global__ __launch_bounds__(256) void causal_conv_strip_kernel(hymeta_causal_conv_args a) {
+  typedef typename A::elem elem;
+  constexpr int MH = HYMETA_CONV_MAX_TAPS - 1;
+  const int t0 = blockIdx.x * kConvRows, t1 = min(t0 + kConvRows, a.num_tokens);
+  const int c = 4 * (blockIdx.y * 256 + threadIdx.x), hist = a.taps - 1;
+  if (blockIdx.y == 0 && a.dt_in != nullptr) {
+    for (int idx = threadIdx.x; idx < (t1 - t0) * a.dt_heads; idx += 256) {
+      const int64_t t = t0 + idx / a.dt_heads;
+      const int hh = idx % a.dt_heads;
+      const float dt = softplus_f(A::ld(static_cast<const elem*>(a.dt_in) + t * a.dt_stride_t + hh) + a.dt_bias[hh]);
+      a.dt_out[t * a.dt_heads + hh] = dt;
+      a.log2_decay_out[t * a.dt_heads + hh] = -expf(a.a_log[hh]) * dt * 1.4426950408889634f;
+    }
+  }
+  if (c >= a.channels) return;
+  float w[HYMETA_CONV_MAX_TAPS][4], bias[4], past[MH][4];
+#pragma unroll
+  for (int j = 0; j < HYMETA_CONV_MAX_TAPS; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[j][e] = j < a.taps ? a.weight[static_cast<int64_t>(c + e) * a.taps + j] : 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) bias[e] = a.bias ? a.bias[c + e] : 0.f;
+  const elem* x = static_cast<const elem*>(a.x);
+  int s = seq_of_row(a.query_start_loc, a.num_seqs, t0);
+  int r0 = a.query_start_loc[s], r1 = a.query_start_loc[s + 1];
+  // past[j]: the input hist - j rows before row t (the oldest first), from the step's rows, the sequence's state, or zeros
+  auto fetch_past = [&](int t) {
+    const int i = t - r0;
+    const int slot = a.slot_idx ? a.slot_idx[s] : -1;
+    const elem* state = (a.conv_state && slot >= 0 && a.context_lens[s] > 0)
+                            ? static_cast<const elem*>(a.conv_state) + static_cast<int64_t>(slot) * hist * a.channels : nullptr;
+#pragma unroll
+    for (int j = 0; j < MH; ++j) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) past[j][e] = 0.f;
+      if (j >= hist) continue;
+      const int back = hist - j;
+      if (back <= i) A::ld4(x + static_cast<int64_t>(t - back) * a.x_stride_t + c, past[j]);
+      else if (state) A::ld4(state + static_cast<int64_t>(hist - (back - i)) * a.channels + c, past[j]);
+    }
+  };
+  fetch_past(t0);
+  for (int t = t0; t < t1; ++t) {
+    if (t >= r1) {
+      while (t >= r1) r1 = a.query_start_loc[++s + 1];
+      r0 = a.query_start_loc[s];
+      fetch_past(t);
+    }
+    float cur[4], acc[4];
+    A::ld4(x + static_cast<int64_t>(t) * a.x_stride_t + c, cur);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = bias[e];
+#pragma unroll
+    for (int j = 0; j < MH; ++j)
+      if (j < hist) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w[j][e], past[j][e], acc[e]);
+      }
+#pragma unroll
+    for (int j = 0; j < HYMETA_CONV_MAX_TAPS; ++j)
+      if (j == hist) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w[j][e], cur[e], acc[e]);
+      }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = acc[e] * sigmoid_exact(acc[e]);
+    A::st4(static_cast<elem*>(a.out) + static_cast<int64_t>(t) * a.channels + c, acc);
+    // the window moves on by a row (in ascending j: past[j + 1] is still the old one)
+#pragma unroll
+    for (int j = 0; j < MH; ++j) {
+      constexpr int kLast = MH - 1;
+      const int nxt = j < kLast ? j + 1 : kLast;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (j + 1 < hist) past[j][e] = past[nxt][e];
+        else if (j + 1 == hist) past[j][e] = cur[e];
+      }
+    }
+  }
+}
+
 // grid = (sequences, channel runs of 256): the state becomes the last taps - 1 input rows (older rows of the old state move
 // up where the step brought fewer rows).  A thread reads all of its channel's old rows before it writes.
 template <typename A>
@@ -209,7 +315,11 @@ extern "C" int hymeta_stream_add_norm(const hymeta_stream_add_norm_args* args, h
   for (int i = 0; i < a.num_terms; ++i)
     if (!a.y[i] || a.y_stride_t[i] < a.width) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
-  const bool cached = a.width <= 256 * kAddPerThread;
+  // runs of four: every pointer and stride in whole fours of its type, the row inside the registers
+  const int eb = a.act_dtype == HYMETA_BF16 ? 2 : 4;
+  bool cached = a.width % 4 == 0 && a.width <= 256 * 4 * kAddVecs && reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && a.x_stride_t % 4 == 0 &&
+                (!a.h_out || reinterpret_cast<uintptr_t>(a.h_out) % (4 * eb) == 0);
+  for (int i = 0; i < a.num_terms; ++i) cached = cached && reinterpret_cast<uintptr_t>(a.y[i]) % (4 * eb) == 0 && a.y_stride_t[i] % 4 == 0;
   if (a.act_dtype == HYMETA_BF16) {
     if (cached) hipLaunchKernelGGL((stream_add_norm_kernel<ActBf16, true>), dim3(a.num_tokens), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((stream_add_norm_kernel<ActBf16, false>), dim3(a.num_tokens), dim3(256), 0, st, a);
@@ -253,8 +363,17 @@ extern "C" int hymeta_causal_conv(const hymeta_causal_conv_args* args, hymeta_st
   if (runs > 65535 || a.num_seqs > 65535) return HYMETA_ERR_UNSUPPORTED;
   hipStream_t st = begin_launches(stream);
   const bool bf = a.act_dtype == HYMETA_BF16;
-  if (bf) hipLaunchKernelGGL(causal_conv_kernel<ActBf16>, dim3(a.num_tokens, runs), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(causal_conv_kernel<ActF32>, dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+  const int eb = bf ? 2 : 4;
+  const bool fours = a.channels % 4 == 0 && a.x_stride_t % 4 == 0 && reinterpret_cast<uintptr_t>(a.x) % (4 * eb) == 0 &&
+                     reinterpret_cast<uintptr_t>(a.out) % (4 * eb) == 0 && (!a.conv_state || reinterpret_cast<uintptr_t>(a.conv_state) % (4 * eb) == 0);
+  if (fours && a.num_tokens >= 4 * kConvRows) {
+    const dim3 grid((a.num_tokens + kConvRows - 1) / kConvRows, (a.channels / 4 + 255) / 256);
+    if (bf) hipLaunchKernelGGL(causal_conv_strip_kernel<ActBf16>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(causal_conv_strip_kernel<ActF32>, grid, dim3(256), 0, st, a);
+  } else {
+    if (bf) hipLaunchKernelGGL(causal_conv_kernel<ActBf16>, dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(causal_conv_kernel<ActF32>, dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+  }
   if (a.conv_state && a.taps > 1) {
     if (bf) hipLaunchKernelGGL(causal_conv_state_kernel<ActBf16>, dim3(a.num_seqs, runs), dim3(256), 0, st, a);
     else hipLaunchKernelGGL(causal_conv_state_kernel<ActF32>, dim3(a.num_seqs, runs), dim3(256), 0, st, a);

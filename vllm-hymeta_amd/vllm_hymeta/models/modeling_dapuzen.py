@@ -225,9 +225,12 @@ class DapuzenForCausalLM(torch.nn.Module, HasInnerState, IsHybrid):
             rows = [act(p + "q", (H * D, W)), act(p + "k", (G * D, W)), act(p + "v", (G * Dv, W))]
             bias = [act(p + "q.b", (H * D,)), act(p + "k.b", (G * D,)), act(p + "v.b", (G * Dv,))] if a.bias else None
             if a.gate:
-                rows.append(act(p + "g", (H, W)))
+                # the gates' rows ride behind the values'; zero rows keep the projection's row a whole number of 16 bytes,
+                # which the matrix-core attention kernels ask of the queries' stride
+                pad = -(sum(r.shape[0] for r in rows) + H) % 8
+                rows.append(torch.cat([act(p + "g", (H, W)), torch.zeros(pad, W, dtype=dt, device=dev)], 0))
                 if bias is not None:
-                    bias.append(torch.zeros(H, dtype=dt, device=dev))
+                    bias.append(torch.zeros(H + pad, dtype=dt, device=dev))
             o = linear([act(p + "o", (W, H * Dv))], [act(p + "o.b", (W,))] if a.bias else None)
             return WindowAttentionMixer(linear(rows, bias), o, m.attn_layers[str(layer)], a.rot_dims, freqs(a), a.gate)
 
