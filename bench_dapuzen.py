@@ -199,7 +199,8 @@ def kernel_table(dev, W, H, G, D, B, ctx, L, E, I, top, ff, window, N=128, P=64)
         cw, cb = rnd(C, 4, std=0.5, dtype=torch.float32).contiguous(), rnd(C, std=0.1, dtype=torch.float32)
         cstate = torch.zeros(max(B, 4), 3, C, dtype=bf, device=dev)
         dtb, alog = torch.zeros(Hs, device=dev), torch.zeros(Hs, device=dev)
-        add(f"causal_conv_silu (+ step sizes) T={T}", lambda: hip_ops.causal_conv_silu(pin[:, :C], cw, cb, cstate, *lay, dt_in=pin[:, C:], dt_bias=dtb, a_log=alog),
+        add(f"causal_conv_silu (+ step sizes) T={T}", lambda: hip_ops.causal_conv_silu(pin[:, :C], cw, cb, cstate, *lay, dt_in=pin[:, C:], dt_bias=dtb, a_log=alog,
+                                                                                          max_query_len=1 if T == B else T),
             nbytes=T * C * 4)
         x = rnd(T, W, dtype=torch.float32)
         wn = 1 + rnd(W, std=0.1, dtype=torch.float32)

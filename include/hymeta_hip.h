@@ -1606,6 +1606,7 @@ typedef struct hymeta_causal_conv_args {
   float* log2_decay_out;       /* [num_tokens, dt_heads] */
   int32_t num_tokens, num_seqs, channels, taps, dt_heads, act_dtype;
   int64_t x_stride_t, dt_stride_t;
+  int32_t single_rows;         /* != 0: the caller knows every sequence brings exactly one row (a decode step): one launch */
 } hymeta_causal_conv_args;
 int hymeta_causal_conv(const hymeta_causal_conv_args* args, hymeta_stream_t stream);
 
@@ -1634,7 +1635,11 @@ typedef struct hymeta_decay_scan_args {
   const int32_t* slot_idx;
   int32_t num_tokens, num_seqs, num_heads, num_qk_heads, head_dim, v_dim, act_dtype, max_query_len;
   int64_t q_stride_t, k_stride_t, v_stride_t;
+  void* workspace;             /* hymeta_decay_scan_workspace_bytes(...) bytes, or NULL when that is 0 */
+  size_t workspace_bytes;
 } hymeta_decay_scan_args;
+/* > 0 for steps with long portions: they run in segments side by side (summarise / chain / apply: three launches). */
+size_t hymeta_decay_scan_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t head_dim, int32_t v_dim, int32_t max_query_len);
 int hymeta_decay_scan(const hymeta_decay_scan_args* args, hymeta_stream_t stream);
 
 #ifdef __cplusplus

@@ -260,7 +260,7 @@ def test_causal_convolution_in_portions_carries_its_inputs(dtype, C, taps, heads
         rows = torch.cat([xs[k][at:at + n] for k, at, n in step]).to(DEV)
         lay = layout_of([n for _, _, n in step], [at for _, at, _ in step], [slots[k] for k, _, _ in step])
         out, dt, ld = hip_ops.causal_conv_silu(rows[:, :C], w.to(DEV), b.to(DEV), state, lay.query_start_loc, lay.context_lens, lay.slot_idx,
-                                               dt_in=rows[:, C:C + heads], dt_bias=dt_bias.to(DEV), a_log=a_log.to(DEV))
+                                               dt_in=rows[:, C:C + heads], dt_bias=dt_bias.to(DEV), a_log=a_log.to(DEV), max_query_len=lay.max_query_len)
         r = 0
         for k, _, n in step:
             dts[k].append(dt[r:r + n])
@@ -269,7 +269,7 @@ def test_causal_convolution_in_portions_carries_its_inputs(dtype, C, taps, heads
         return out
 
     # (the last step: a sequence that ends inside a strip of rows, the next one starting there with a state of its own)
-    got = in_steps(lens, [[(0, 2)], [(0, 1), (1, 1)], [(0, 1), (2, 4)], [(0, 3), (2, 1)], [(2, 7), (0, 30)], [(0, 53), (2, 33)]], run)
+    got = in_steps(lens, [[(0, 2)], [(0, 1), (1, 1)], [(0, 1), (2, 4)], [(0, 3), (2, 1)], [(0, 1), (2, 1)], [(2, 6), (0, 29)], [(0, 53), (2, 33)]], run)
     tol = 2e-6 if dtype == torch.float32 else 6e-3
     for k in lens:
         assert rel_err(got[k], refs[k]) < tol, k
@@ -340,6 +340,41 @@ def test_decayed_scan_in_portions_and_single_rows(dtype, H, G, D, P, per_token):
     ref = _scan_ref(torch.cat([qs[0], q1]).double(), torch.cat([ks[0], k1]).double(), torch.cat([vs[0], v1]).double(),
                     torch.cat([lds[0], lds[0][:1]]).double(), torch.cat([bs[0], bs[0][:1]]).double(), skip.double())[-1:]
     assert rel_err(more, ref) < 4 * tol
+
+
+@pytest.mark.parametrize("per_token", [False, True])
+def test_decayed_scan_of_a_long_portion_in_segments(per_token):
+    """A portion long enough to run as segments side by side (bf16, matrix-core sizes) beside a short one, after a carried
+    state: the same rows as the chunks one after the other, and as the plain recurrence."""
+    from vllm_hymeta import hip_ops
+    g = torch.Generator().manual_seed(11)
+    H, G, D, P = 2, 1, 64, 32
+    lens = {0: 2700, 1: 40}
+    dtype = torch.bfloat16
+    qs = {k: (torch.randn(n, G, D, generator=g) * D ** -0.25).to(dtype) for k, n in lens.items()}
+    ks = {k: (torch.randn(n, G, D, generator=g) * D ** -0.25).to(dtype) for k, n in lens.items()}
+    vs = {k: torch.randn(n, H, P, generator=g).to(dtype) for k, n in lens.items()}
+    decay = torch.tensor([0.97, 0.999])
+    lds = {k: (-torch.rand(n, H, generator=g) * 0.1) if per_token else torch.log2(decay).expand(n, H).contiguous() for k, n in lens.items()}
+    bs = {k: (torch.rand(n, H, generator=g) + 0.2) if per_token else torch.ones(n, H) for k, n in lens.items()}
+    skip = torch.randn(H, generator=g) if per_token else torch.zeros(H)
+    refs = {k: _scan_ref(qs[k].double(), ks[k].double(), vs[k].double(), lds[k].double(), bs[k].double(), skip.double()) for k in lens}
+    state = torch.full((2, H, D, P), 3.0, dtype=torch.float32, device=DEV)
+
+    def run(step):
+        cat = lambda d: torch.cat([d[k][at:at + n] for k, at, n in step]).to(DEV)      # noqa: E731
+        lay = layout_of([n for _, _, n in step], [at for _, at, _ in step], [k for k, _, _ in step])
+        kw = dict(log2_decay=cat(lds), v_scale=cat(bs), skip=skip.to(DEV)) if per_token else dict(decay=decay.to(DEV))
+        return hip_ops.decay_scan(cat(qs), cat(ks), cat(vs), state, lay.query_start_loc, lay.context_lens, lay.slot_idx, lay.max_query_len, **kw)
+
+    got = in_steps(lens, [[(0, 100)], [(0, 2600), (1, 40)]], run)            # 2600 rows from a carried state: three segments
+    for k in lens:
+        assert rel_err(got[k], refs[k]) < 6e-3, k
+    end = state.clone()
+    got = in_steps(lens, [[(0, 1500)], [(0, 1200), (1, 40)]], run)           # below the segments' threshold: chunk after chunk
+    assert rel_err(state, end) < 1e-4
+    for k in lens:
+        assert rel_err(got[k], refs[k]) < 6e-3, k
 
 
 def test_state_space_recurrence_is_the_scan_with_its_step_sizes():

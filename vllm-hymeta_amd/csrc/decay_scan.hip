@@ -145,20 +145,33 @@ __global__ __launch_bounds__(256) void decay_scan_step_kernel(hymeta_decay_scan_
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int kChunk = HYMETA_SCAN_CHUNK, kSliceV = 32;
 constexpr int kChunkMinRows = 8;            // shorter portions go token by token
+// Steps with a portion of kSegmentMinRows or more are cut into segments of kSegmentRows that run side by side: every
+// segment but the last is summarised from a zero state (its state and the sum of its log2 decays), the summaries are chained
+// into the states in front of the segments, then every segment runs from its state (three launches; a sequence's chunks
+// otherwise follow each other in one workgroup per head and value slice, which leaves most of the chip idle under a single
+// long prompt).
+constexpr int kSegmentRows = 1024, kSegmentMinRows = 2048;
+enum ChunkMode { kWhole = 0, kSummarise = 1, kApply = 2 };
 constexpr float kMinLog2 = -1.0e4f;         // a decay of 0 (or an overflowed step size): finite, so that differences of sums stay numbers
 
 __device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 
 template <int D>
-__global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan_args a, int min_rows) {
+__global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan_args a, int min_rows, int seg_rows, int nseg, int mode) {
   constexpr int PK = D + 8, PT = kChunk + 8, NBW = (2 * D / 16) / 4;
   __shared__ __attribute__((aligned(16))) uint16_t sk[kChunk * PK];          // k, a row per key
   __shared__ __attribute__((aligned(16))) uint16_t skt[2][D * PT];           // decayed keys, transposed [d][key], hi / lo
   __shared__ __attribute__((aligned(16))) uint16_t svt[kSliceV * PT];        // v of the slice, transposed [c][key]
   __shared__ __attribute__((aligned(16))) uint16_t sst[2][kSliceV * PK];     // state^T [c][d], hi / lo
-  const int h = blockIdx.x, s = blockIdx.y, vs = blockIdx.z;
-  const int r0 = a.query_start_loc[s], rows = a.query_start_loc[s + 1] - r0;
-  if (rows < min_rows) return;
+  const int h = blockIdx.x, s = blockIdx.y / nseg, seg = blockIdx.y % nseg, vs = blockIdx.z;
+  const int r0 = a.query_start_loc[s], rows_all = a.query_start_loc[s + 1] - r0;
+  if (rows_all < min_rows) return;
+  // this workgroup's rows of the portion: all of them (kWhole), or one segment
+  const int r_lo = mode == kWhole ? 0 : seg * seg_rows;
+  if (r_lo >= rows_all) return;
+  const int rows = mode == kWhole ? rows_all : min(rows_all, r_lo + seg_rows);        // (end of the rows, not their count)
+  const bool last = rows == rows_all;
+  if (mode == kSummarise && last) return;                    // nothing comes behind the last segment
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g4 = lane >> 4;
   const int H = a.num_heads, Dv = a.v_dim;
   const int g = h / (H / a.num_qk_heads);
@@ -167,12 +180,18 @@ __global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan
   const float l2_const = a.decay ? fmaxf(a.decay[h] > 0.f ? log2f(a.decay[h]) : -INFINITY, kMinLog2) : 0.f;
   const float skip = a.skip ? a.skip[h] : 0.f;
   const bool carry = st != nullptr && a.context_lens[s] > 0;
+  // a segment's place in the workspace: its summary (kSummarise writes it), then the state in front of it (kApply reads it);
+  // the segments' sums of log2 decays lie behind all the states
+  const int64_t seg_at = (static_cast<int64_t>(s) * nseg + seg) * H + h;
+  float* wsp = mode == kWhole ? nullptr : static_cast<float*>(a.workspace) + (seg_at * D) * Dv + vs * kSliceV;
+  const float* init = mode == kWhole ? (carry ? st : nullptr) : mode == kApply ? wsp : nullptr;
   f32x4v S[NBW];
 #pragma unroll
   for (int ib = 0; ib < NBW; ++ib) {
     const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
-    S[ib] = carry ? *reinterpret_cast<const f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) : f32x4v{0.f, 0.f, 0.f, 0.f};
+    S[ib] = init ? *reinterpret_cast<const f32x4v*>(init + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) : f32x4v{0.f, 0.f, 0.f, 0.f};
   }
+  float seg_total = 0.f;
   auto state_to_lds = [&]() {
 #pragma unroll
     for (int ib = 0; ib < NBW; ++ib) {
@@ -214,7 +233,7 @@ __global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan
 #pragma unroll
     for (int sd = 0; sd < D / 32; ++sd) {
       rq[sd] = u32x4{0u, 0u, 0u, 0u};
-      if (i < nrow) rq[sd] = ld16g(qp + (t0 + i) * a.q_stride_t + 32 * sd + 8 * g4);
+      if (i < nrow && mode != kSummarise) rq[sd] = ld16g(qp + (t0 + i) * a.q_stride_t + 32 * sd + 8 * g4);
     }
     rl = 0.f, rb = 0.f;
     if (lane < nrow) {
@@ -223,8 +242,8 @@ __global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan
     }
   };
   static_assert(kChunk * (kSliceV / 8) == 256, "one group of the value slice per thread");
-  fetch(0);
-  for (int c0 = 0; c0 < rows; c0 += kChunk) {
+  fetch(r_lo);
+  for (int c0 = r_lo; c0 < rows; c0 += kChunk) {
     const int nrow = min(kChunk, rows - c0);
     // running sums of the chunk's log2 decays over the wave's lanes (rows past the portion add 0)
     float cum = rl;
@@ -234,6 +253,7 @@ __global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan
       if (lane >= o) cum += up;
     }
     const float total = __shfl(cum, nrow - 1, 64);
+    seg_total += total;
     const float bw = rb;
     // a wave's lanes hold 64 different rows of one 8-column group (row = lane): the transposed 2-byte stores of a wave fall
     // on consecutive addresses, the row-major 16-byte stores on different banks
@@ -262,7 +282,7 @@ __global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan
     for (int sd = 0; sd < D / 32; ++sd) q[sd] = __builtin_bit_cast(bf16x8, rq[sd]);
     __syncthreads();
     if (c0 + kChunk < rows) fetch(c0 + kChunk);        // in flight while this chunk is multiplied
-    {
+    if (mode != kSummarise) {
       // weights of the chunk's own rows: (q_i . k_j) 2^(c_i - c_j) b_j for j <= i, as hi + lo parts
       const float cum_i = __shfl(cum, i, 64);
       uint32_t phi[4][2], plo[4][2];
@@ -339,12 +359,41 @@ __global__ __launch_bounds__(256) void decay_scan_chunk_kernel(hymeta_decay_scan
     __syncthreads();            // every wave is done with this chunk's tiles and with the old state's image
     state_to_lds();             // (made visible by the barrier after the next chunk's staging)
   }
-  if (st != nullptr) {
+  float* to = mode == kSummarise ? wsp : (last ? st : nullptr);
+  if (to != nullptr) {
 #pragma unroll
     for (int ib = 0; ib < NBW; ++ib) {
       const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
-      *reinterpret_cast<f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) = S[ib];
+      *reinterpret_cast<f32x4v*>(to + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) = S[ib];
     }
+  }
+  if (mode == kSummarise && vs == 0 && tid == 0) {
+    float* totals = static_cast<float*>(a.workspace) + static_cast<int64_t>(a.num_seqs) * nseg * H * D * Dv;
+    totals[seg_at] = seg_total;
+  }
+}
+
+// The segments' summaries (each segment's state had it started from zero) become the states in front of the segments:
+// run = carried state; per segment: place <- run, run <- 2^(segment's sum of log2 decays) run + summary.  An element per thread.
+__global__ __launch_bounds__(256) void decay_scan_chain_kernel(hymeta_decay_scan_args a, int min_rows, int seg_rows, int nseg) {
+  const int s = blockIdx.y;
+  const int rows = a.query_start_loc[s + 1] - a.query_start_loc[s];
+  if (rows < min_rows) return;
+  const int64_t per_head = static_cast<int64_t>(a.head_dim) * a.v_dim, per_seq = per_head * a.num_heads;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= per_seq) return;
+  const int h = static_cast<int>(idx / per_head);
+  const int slot = a.slot_idx[s];
+  float run = (slot >= 0 && a.context_lens[s] > 0) ? a.state[static_cast<int64_t>(slot) * per_seq + idx] : 0.f;
+  const int segs = (rows + seg_rows - 1) / seg_rows;
+  float* p = static_cast<float*>(a.workspace) + static_cast<int64_t>(s) * nseg * per_seq + idx;
+  const float* totals = static_cast<const float*>(a.workspace) + static_cast<int64_t>(a.num_seqs) * nseg * per_seq +
+                        static_cast<int64_t>(s) * nseg * a.num_heads + h;
+  for (int seg = 0; seg < segs; ++seg, p += per_seq) {
+    const bool more = seg < segs - 1;
+    const float summary = more ? *p : 0.f;
+    *p = run;
+    if (more) run = __builtin_amdgcn_exp2f(totals[static_cast<int64_t>(seg) * a.num_heads]) * run + summary;
   }
 }
 
@@ -378,6 +427,12 @@ void launch_rows(const hymeta_decay_scan_args& a, hipStream_t st, int min_rows, 
 
 using namespace hymeta;
 
+extern "C" size_t hymeta_decay_scan_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t head_dim, int32_t v_dim, int32_t max_query_len) {
+  if (num_seqs <= 0 || num_heads <= 0 || head_dim <= 0 || v_dim <= 0 || max_query_len < kSegmentMinRows) return 0;
+  const size_t nseg = (static_cast<size_t>(max_query_len) + kSegmentRows - 1) / kSegmentRows;
+  return nseg * num_seqs * num_heads * (static_cast<size_t>(head_dim) * v_dim + 1) * sizeof(float);
+}
+
 extern "C" int hymeta_decay_scan(const hymeta_decay_scan_args* args, hymeta_stream_t stream) {
   if (!args_ok(args)) return HYMETA_ERR_INVALID_ARG;
   const hymeta_decay_scan_args& a = *args;
@@ -393,10 +448,25 @@ extern "C" int hymeta_decay_scan(const hymeta_decay_scan_args* args, hymeta_stre
   hipStream_t st = begin_launches(stream);
   int max_rows = 0x7fffffff;
   if (chunk_shape(a) && a.max_query_len >= kChunkMinRows) {
-    const dim3 grid(a.num_heads, a.num_seqs, a.v_dim / kSliceV);
-    if (a.head_dim == 32) hipLaunchKernelGGL(decay_scan_chunk_kernel<32>, grid, dim3(256), 0, st, a, kChunkMinRows);
-    else if (a.head_dim == 64) hipLaunchKernelGGL(decay_scan_chunk_kernel<64>, grid, dim3(256), 0, st, a, kChunkMinRows);
-    else hipLaunchKernelGGL(decay_scan_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    const size_t need = hymeta_decay_scan_workspace_bytes(a.num_seqs, a.num_heads, a.head_dim, a.v_dim, a.max_query_len);
+    const int nseg = need > 0 ? (a.max_query_len + kSegmentRows - 1) / kSegmentRows : 1;
+    if (need > 0 && (!a.workspace || a.workspace_bytes < need)) return HYMETA_ERR_WORKSPACE;
+    if (static_cast<int64_t>(a.num_seqs) * nseg > 65535) return HYMETA_ERR_UNSUPPORTED;
+    const dim3 grid(a.num_heads, a.num_seqs * nseg, a.v_dim / kSliceV);
+    auto chunks = [&](int mode) {
+      if (a.head_dim == 32) hipLaunchKernelGGL(decay_scan_chunk_kernel<32>, grid, dim3(256), 0, st, a, kChunkMinRows, kSegmentRows, nseg, mode);
+      else if (a.head_dim == 64) hipLaunchKernelGGL(decay_scan_chunk_kernel<64>, grid, dim3(256), 0, st, a, kChunkMinRows, kSegmentRows, nseg, mode);
+      else hipLaunchKernelGGL(decay_scan_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows, kSegmentRows, nseg, mode);
+    };
+    if (nseg == 1) {
+      chunks(kWhole);
+    } else {
+      chunks(kSummarise);
+      const int64_t per_seq = static_cast<int64_t>(a.num_heads) * a.head_dim * a.v_dim;
+      hipLaunchKernelGGL(decay_scan_chain_kernel, dim3(static_cast<unsigned>((per_seq + 255) / 256), a.num_seqs), dim3(256), 0, st, a, kChunkMinRows,
+                         kSegmentRows, nseg);
+      chunks(kApply);
+    }
     max_rows = kChunkMinRows - 1;
   }
   int min_rows = 1;

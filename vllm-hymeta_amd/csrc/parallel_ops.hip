@@ -154,11 +154,13 @@ __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + lo
 
 // grid = (tokens, channel runs of 256): a thread computes one channel of one row from the row and its taps - 1
 // predecessors (rows of the step, or the sequence's state).  The first run's workgroup also computes the row's step sizes.
-template <typename A>
+// SingleRows: every sequence brings one row (row t is sequence t's), and the thread that read its channel of the state
+// also moves it on by the row -- a decode step's convolution in one launch.
+template <typename A, bool SingleRows>
 __global__ __launch_bounds__(256) void causal_conv_kernel(hymeta_causal_conv_args a) {
   typedef typename A::elem elem;
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
-  const int s = seq_of_row(a.query_start_loc, a.num_seqs, t);
+  const int s = SingleRows ? t : seq_of_row(a.query_start_loc, a.num_seqs, t);
   const int r0 = a.query_start_loc[s], i = t - r0, hist = a.taps - 1;
   if (blockIdx.y == 0 && a.dt_in != nullptr && threadIdx.x < a.dt_heads) {
     const int h = threadIdx.x;
@@ -171,18 +173,22 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(hymeta_causal_conv_arg
   }
   if (c >= a.channels) return;
   const int slot = a.slot_idx ? a.slot_idx[s] : -1;
-  const elem* state = (a.conv_state && slot >= 0 && a.context_lens[s] > 0)
-                          ? static_cast<const elem*>(a.conv_state) + static_cast<int64_t>(slot) * hist * a.channels : nullptr;
+  elem* own = (a.conv_state && slot >= 0) ? static_cast<elem*>(a.conv_state) + static_cast<int64_t>(slot) * hist * a.channels : nullptr;
+  const elem* state = a.context_lens[s] > 0 ? own : nullptr;
   const elem* x = static_cast<const elem*>(a.x);
   float acc = a.bias ? a.bias[c] : 0.f;
+  elem taps_in[HYMETA_CONV_MAX_TAPS];                 // the inputs as stored (what the state keeps)
   for (int j = 0; j < a.taps; ++j) {
     const int back = hist - j;                    // rows before t
-    float v = 0.f;
-    if (back <= i) v = A::ld(x + static_cast<int64_t>(t - back) * a.x_stride_t + c);
-    else if (state) v = A::ld(state + static_cast<int64_t>(hist - (back - i)) * a.channels + c);       // state row hist - 1 is the newest
-    acc = fmaf(a.weight[static_cast<int64_t>(c) * a.taps + j], v, acc);
+    elem raw = static_cast<elem>(0);
+    if (back <= i) raw = x[static_cast<int64_t>(t - back) * a.x_stride_t + c];
+    else if (state) raw = state[static_cast<int64_t>(hist - (back - i)) * a.channels + c];       // state row hist - 1 is the newest
+    taps_in[j] = raw;
+    acc = fmaf(a.weight[static_cast<int64_t>(c) * a.taps + j], A::ld(&raw), acc);
   }
   A::st(static_cast<elem*>(a.out) + static_cast<int64_t>(t) * a.channels + c, acc * sigmoid_exact(acc));
+  if (SingleRows && own != nullptr)
+    for (int j = 0; j < hist; ++j) own[static_cast<int64_t>(j) * a.channels + c] = taps_in[j + 1];
 }
 
 // Many rows, channels in whole fours: a thread takes four consecutive channels through a strip of kConvRows rows, the
@@ -370,9 +376,13 @@ extern "C" int hymeta_causal_conv(const hymeta_causal_conv_args* args, hymeta_st
     const dim3 grid((a.num_tokens + kConvRows - 1) / kConvRows, (a.channels / 4 + 255) / 256);
     if (bf) hipLaunchKernelGGL(causal_conv_strip_kernel<ActBf16>, grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL(causal_conv_strip_kernel<ActF32>, grid, dim3(256), 0, st, a);
+  } else if (a.num_tokens == a.num_seqs && a.single_rows) {
+    if (bf) hipLaunchKernelGGL((causal_conv_kernel<ActBf16, true>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((causal_conv_kernel<ActF32, true>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+    return launch_status();
   } else {
-    if (bf) hipLaunchKernelGGL(causal_conv_kernel<ActBf16>, dim3(a.num_tokens, runs), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(causal_conv_kernel<ActF32>, dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+    if (bf) hipLaunchKernelGGL((causal_conv_kernel<ActBf16, false>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((causal_conv_kernel<ActF32, false>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
   }
   if (a.conv_state && a.taps > 1) {
     if (bf) hipLaunchKernelGGL(causal_conv_state_kernel<ActBf16>, dim3(a.num_seqs, runs), dim3(256), 0, st, a);

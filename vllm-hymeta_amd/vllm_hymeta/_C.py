@@ -553,6 +553,7 @@ class CausalConvArgs(_Args):
         ("dt_in", _ptr), ("dt_bias", _ptr), ("a_log", _ptr), ("dt_out", _ptr), ("log2_decay_out", _ptr),
         ("num_tokens", _i32), ("num_seqs", _i32), ("channels", _i32), ("taps", _i32), ("dt_heads", _i32), ("act_dtype", _i32),
         ("x_stride_t", _i64), ("dt_stride_t", _i64),
+        ("single_rows", _i32),
     ]
 
 
@@ -564,6 +565,7 @@ class DecayScanArgs(_Args):
         ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("num_qk_heads", _i32), ("head_dim", _i32), ("v_dim", _i32),
         ("act_dtype", _i32), ("max_query_len", _i32),
         ("q_stride_t", _i64), ("k_stride_t", _i64), ("v_stride_t", _i64),
+        ("workspace", _ptr), ("workspace_bytes", _sz),
     ]
 
 
@@ -660,6 +662,7 @@ _SIGNATURES = {
     "hymeta_stream_add_norm": (C.c_int, [C.POINTER(StreamAddNormArgs), _ptr]),
     "hymeta_rotary_cache": (C.c_int, [C.POINTER(RotaryCacheArgs), _ptr]),
     "hymeta_causal_conv": (C.c_int, [C.POINTER(CausalConvArgs), _ptr]),
+    "hymeta_decay_scan_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),
     "hymeta_decay_scan": (C.c_int, [C.POINTER(DecayScanArgs), _ptr]),
 }
 

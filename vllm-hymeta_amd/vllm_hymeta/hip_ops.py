@@ -2258,12 +2258,13 @@ def rotary_cache_(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
 
 def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], conv_state: Optional[torch.Tensor],
                      query_start_loc: torch.Tensor, context_lens: torch.Tensor, slot_idx: Optional[torch.Tensor],
-                     dt_in: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None, a_log: Optional[torch.Tensor] = None):
+                     dt_in: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None, a_log: Optional[torch.Tensor] = None,
+                     max_query_len: Optional[int] = None):
     """``silu(bias + sum_j weight[:, j] x[t - taps + 1 + j])`` per channel over each sequence's rows of ``x [T, C]`` (a view
     with any row stride); ``weight`` fp32 ``[C, taps]``; ``conv_state [slots, taps - 1, C]`` (x's type) carries a sequence's
     last input rows between steps, in place.  With ``dt_in [T, heads]`` also returns fp32 ``softplus(dt_in + dt_bias)`` and
-    ``-exp(a_log) dt log2(e)``, both ``[T, heads]``: a state-space layer's step sizes and log2 decays.  Returns ``out`` or
-    ``(out, dt, log2_decay)``."""
+    ``-exp(a_log) dt log2(e)``, both ``[T, heads]``: a state-space layer's step sizes and log2 decays.  ``max_query_len`` 1
+    (every sequence brings one row): the state moves on in the same launch.  Returns ``out`` or ``(out, dt, log2_decay)``."""
     _dev(x, weight, bias, conv_state, query_start_loc, context_lens, slot_idx, dt_in, dt_bias, a_log)
     _require(x.dim() == 2 and x.stride(1) == 1 and x.dtype in _DT, "x must be row-contiguous [T, C], bf16 or fp32")
     T, Cn = x.shape
@@ -2279,6 +2280,7 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     a.x, a.weight, a.bias, a.out = _p(x), _p(weight), _p(bias), _p(out)
     a.query_start_loc, a.context_lens = _p(query_start_loc), _p(context_lens)
     a.num_tokens, a.num_seqs, a.channels, a.taps, a.act_dtype, a.x_stride_t = T, S, Cn, taps, _act(x), x.stride(0)
+    a.single_rows = int(max_query_len == 1 and T == S)
     if conv_state is not None and taps > 1:
         _require(slot_idx is not None, "conv_state needs slot_idx")
         _i32vec(slot_idx, S, "slot_idx")
@@ -2332,5 +2334,10 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.T
     a.num_tokens, a.num_seqs, a.num_heads, a.num_qk_heads, a.head_dim, a.v_dim = T, S, H, Hqk, D, Dv
     a.act_dtype, a.max_query_len = _act(q), max_query_len
     a.q_stride_t, a.k_stride_t, a.v_stride_t = q.stride(0), k.stride(0), v.stride(0)
-    _C.check(_C.load().hymeta_decay_scan(C.byref(a), _stream(q)), "hymeta_decay_scan")
+    lib = _C.load()
+    nbytes = int(lib.hymeta_decay_scan_workspace_bytes(S, H, D, Dv, max_query_len))
+    if nbytes:
+        ws = _workspace(q.device, nbytes, "decay_scan")
+        a.workspace, a.workspace_bytes = _p(ws), ws.numel()
+    _C.check(lib.hymeta_decay_scan(C.byref(a), _stream(q)), "hymeta_decay_scan")
     return out

@@ -44,7 +44,8 @@ class StateSpaceMixer(torch.nn.Module):
         proj = self.in_proj(h)
         xbc, dt, log2_decay = hip_ops.causal_conv_silu(proj[:, inner:inner + ch], self.conv_weight, self.conv_bias, conv_state,
                                                        layout.query_start_loc, layout.context_lens, layout.slot_idx,
-                                                       dt_in=proj[:, inner + ch:inner + ch + H], dt_bias=self.dt_bias, a_log=self.a_log)
+                                                       dt_in=proj[:, inner + ch:inner + ch + H], dt_bias=self.dt_bias, a_log=self.a_log,
+                                                       max_query_len=layout.max_query_len)
         x = xbc[:, :inner].view(-1, H, P)
         b, c = xbc[:, inner:inner + G * N].view(-1, G, N), xbc[:, inner + G * N:].view(-1, G, N)
         y = hip_ops.decay_scan(c, b, x, ssm_state, layout.query_start_loc, layout.context_lens, layout.slot_idx, layout.max_query_len,
