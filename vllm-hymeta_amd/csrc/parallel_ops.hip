@@ -372,14 +372,16 @@ extern "C" int hymeta_causal_conv(const hymeta_causal_conv_args* args, hymeta_st
   const int eb = bf ? 2 : 4;
   const bool fours = a.channels % 4 == 0 && a.x_stride_t % 4 == 0 && reinterpret_cast<uintptr_t>(a.x) % (4 * eb) == 0 &&
                      reinterpret_cast<uintptr_t>(a.out) % (4 * eb) == 0 && (!a.conv_state || reinterpret_cast<uintptr_t>(a.conv_state) % (4 * eb) == 0);
-  if (fours && a.num_tokens >= 4 * kConvRows) {
-    const dim3 grid((a.num_tokens + kConvRows - 1) / kConvRows, (a.channels / 4 + 255) / 256);
-    if (bf) hipLaunchKernelGGL(causal_conv_strip_kernel<ActBf16>, grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(causal_conv_strip_kernel<ActF32>, grid, dim3(256), 0, st, a);
-  } else if (a.num_tokens == a.num_seqs && a.single_rows) {
+  if (a.num_tokens == a.num_seqs && a.single_rows) {
     if (bf) hipLaunchKernelGGL((causal_conv_kernel<ActBf16, true>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((causal_conv_kernel<ActF32, true>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
     return launch_status();
+  }
+  // strips pay once there are rows enough to fill the chip with a quarter of the threads
+  if (fours && a.num_tokens >= 32 * kConvRows) {
+    const dim3 grid((a.num_tokens + kConvRows - 1) / kConvRows, (a.channels / 4 + 255) / 256);
+    if (bf) hipLaunchKernelGGL(causal_conv_strip_kernel<ActBf16>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(causal_conv_strip_kernel<ActF32>, grid, dim3(256), 0, st, a);
   } else {
     if (bf) hipLaunchKernelGGL((causal_conv_kernel<ActBf16, false>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((causal_conv_kernel<ActF32, false>), dim3(a.num_tokens, runs), dim3(256), 0, st, a);
