@@ -225,13 +225,20 @@ def kernel_table(dev, W, H, G, D, B, ctx, L, E, I, top, ff, window, N=128, P=64)
     rows_g = rnd(E + I + 1, W, std=W ** -0.5, dtype=torch.float32)
     corr = rnd(E + I, std=0.01, dtype=torch.float32)
     choice = hip_ops.GroupedChoice(corr, (E + I) // 4, 2, I, 1)
+    rows_0 = rows_g[:E + 1].contiguous()
+    choice_0 = hip_ops.GroupedChoice(corr[:E].contiguous(), max(E // 4, 1), max(E // 4, 1), 0, 1)
     for T in (B, L):
         xm = rnd(T, W)
         wbytes = min(E, T * top) * 3 * ff * W * 2
         fl = T * top * 3 * ff * W * 2
-        add(f"moe_routed_forward grouped softmax, silu experts T={T} (E={E} + {I} identity, top {top})",
-            lambda: hip_ops.moe_routed_forward(xm, rows_g, None, w13, w2, top, hip_ops.ROUTE_SOFTMAX_GROUPED, 1.0, "silu_glu", choice=choice),
+        # like for like: every chosen output is an expert with matrices
+        add(f"moe_routed_forward grouped softmax, silu experts T={T} (E={E}, no identity experts, top {top})",
+            lambda: hip_ops.moe_routed_forward(xm, rows_0, None, w13, w2, top, hip_ops.ROUTE_SOFTMAX_GROUPED, 1.0, "silu_glu", choice=choice_0),
             nbytes=wbytes, flops=fl, iters=10 if T > 256 else 20)
+        # as the model runs it: with random router rows E / (E + I) of the chosen outputs have matrices, the others cost nothing
+        add(f"moe_routed_forward grouped softmax, silu experts T={T} (E={E} + {I} identity, top {top}; flops of the expected {E}/{E + I} share)",
+            lambda: hip_ops.moe_routed_forward(xm, rows_g, None, w13, w2, top, hip_ops.ROUTE_SOFTMAX_GROUPED, 1.0, "silu_glu", choice=choice),
+            nbytes=wbytes, flops=fl * E // (E + I), iters=10 if T > 256 else 20)
         add(f"moe_sigmoid_forward (Geponex) T={T} (E={E}, top {top})", lambda: hip_ops.moe_sigmoid_forward(xm, router, w13, w2, top, 1.0, 7.0), nbytes=wbytes,
             flops=fl, iters=10 if T > 256 else 20)
     return rows
